@@ -83,6 +83,72 @@ void normed_rope_store_kernel(const TA* __restrict__ qkv, const TW* __restrict__
     }
 }
 
+// ---- bias, rotation, then a norm without a weight, cache write ------------------------------------------
+// What another family of designs does with its heads: the projections' biases are added, q and k are turned (in halves,
+// style 1, or in neighbouring pairs, style 2: element 2i with 2i + 1), and only then every query and key head is divided
+// by its root mean square (normed != 0; no weight).  A wave per head of a token, as above; a lane keeps its elements
+// (up to AM_MAX_D / 64) between the sum of squares and the store.
+template <typename TA, typename TB>
+__global__ __launch_bounds__(AM_WAVES * TQK_WAVE)
+void rope_norm_store_kernel(const TA* __restrict__ qkv, const TB* __restrict__ bias, const float* __restrict__ cos_table,
+                            const float* __restrict__ sin_table, int rot_dim, int style, int max_positions, int normed, float eps,
+                            const int32_t* __restrict__ tok_seq, const int32_t* __restrict__ tok_pos, const int32_t* __restrict__ page_table,
+                            int table_width, TA* __restrict__ keys, TA* __restrict__ values, TA* __restrict__ q_out, int n_heads, int n_kv_heads,
+                            int dk, int dv, int write_kv) {
+    const int t = blockIdx.x;
+    const int head = blockIdx.y * AM_WAVES + threadIdx.x / TQK_WAVE;
+    const int lane = threadIdx.x % TQK_WAVE;
+    if (head >= n_heads + 2 * n_kv_heads) return;
+    const int pos = tok_pos[t];
+    const int kind = head < n_heads ? 0 : (head < n_heads + n_kv_heads ? 1 : 2);
+    if (kind != 0 && !write_kv) return;
+    const size_t total = (size_t)(n_heads + n_kv_heads) * dk + (size_t)n_kv_heads * dv;
+    const TA* row = qkv + (size_t)t * total;
+    int page = -1;
+    if (kind != 0) {
+        page = page_table[(size_t)tok_seq[t] * table_width + pos / TQK_PAGE];
+        if (page < 0) return;                          // the host never lets this happen
+    }
+    if (kind == 2) {
+        const int g = head - n_heads - n_kv_heads;
+        const size_t off = (size_t)(n_heads + n_kv_heads) * dk + (size_t)g * dv;
+        TA* dst = values + ((size_t)page * n_kv_heads + g) * TQK_PAGE * dv + value_place(pos % TQK_PAGE);
+        for (int i = lane; i < dv; i += TQK_WAVE)
+            dst[(size_t)i * TQK_PAGE] = from_float<TA>(to_float(row[off + i]) + (bias ? to_float(bias[off + i]) : 0.f));
+        return;
+    }
+    const size_t off = (size_t)head * dk;
+    const int half = rot_dim / 2;
+    const bool rotate = rot_dim > 0 && style != 0 && pos < max_positions;
+    float x[AM_MAX_D / TQK_WAVE];
+    float ss = 0.f;
+#pragma unroll
+    for (int k = 0; k < AM_MAX_D / TQK_WAVE; ++k) {
+        const int i = lane + k * TQK_WAVE;
+        x[k] = 0.f;
+        if (i >= dk) continue;
+        float v = to_float(row[off + i]) + (bias ? to_float(bias[off + i]) : 0.f);
+        if (rotate && i < rot_dim) {
+            const bool first = style == 2 ? (i & 1) == 0 : i < half;
+            const int partner = style == 2 ? (i ^ 1) : (first ? i + half : i - half);
+            const int p = style == 2 ? i / 2 : (first ? i : i - half);
+            const float y = to_float(row[off + partner]) + (bias ? to_float(bias[off + partner]) : 0.f);
+            const float c = cos_table[(size_t)pos * half + p], s = sin_table[(size_t)pos * half + p];
+            v = first ? v * c - y * s : v * c + y * s;
+        }
+        x[k] = v;
+        ss = fmaf(v, v, ss);
+    }
+    const float inv = normed ? 1.f / sqrtf(wave_sum(ss) / (float)dk + eps) : 1.f;
+    TA* dst = kind == 0 ? q_out + ((size_t)t * n_heads + head) * dk
+                        : keys + (((size_t)page * n_kv_heads + (head - n_heads)) * TQK_PAGE + pos % TQK_PAGE) * dk;
+#pragma unroll
+    for (int k = 0; k < AM_MAX_D / TQK_WAVE; ++k) {
+        const int i = lane + k * TQK_WAVE;
+        if (i < dk) dst[i] = from_float<TA>(x[k] * inv);
+    }
+}
+
 // The same for steps of many tokens in bfloat16 (head sizes multiples of 8, half the rotated elements too), in two launches.
 // Queries and keys: a block per token, a thread per 8 neighbouring elements (16 bytes a load and a store); the sums of squares of a
 // head's pieces meet in LDS; the piece a rotated one turns with is read once more (it is in the caches).
@@ -333,6 +399,32 @@ extern "C" int tqk_normed_rope_store(const void* qkv, int act_dtype, const void*
     else return tqk_fail("tqk_normed_rope_store: unknown dtypes %d, %d", act_dtype, w_dtype);
 #undef TQK_NRS
     return tqk_check_launch("tqk_normed_rope_store");
+}
+
+extern "C" int tqk_rope_norm_store(const void* qkv, int act_dtype, const void* bias, int bias_dtype, const float* cos_table, const float* sin_table,
+                                   int rot_dim, int style, int max_positions, int normed, float eps, const int32_t* tok_seq, const int32_t* tok_pos,
+                                   const int32_t* page_table, int table_width, void* keys, void* values, void* q_out, int n_tokens, int n_heads,
+                                   int n_kv_heads, int key_dim, int value_dim, int write_kv, void* stream) {
+    TQK_REQUIRE(qkv && tok_pos && q_out, "tqk_rope_norm_store: null pointer");
+    TQK_REQUIRE(n_tokens >= 0 && n_heads > 0 && n_kv_heads > 0 && key_dim > 0 && value_dim > 0, "tqk_rope_norm_store: bad sizes");
+    TQK_REQUIRE(key_dim <= AM_MAX_D, "tqk_rope_norm_store: heads of %d values, the kernel takes up to %d", key_dim, AM_MAX_D);
+    TQK_REQUIRE(style >= 0 && style <= 2, "tqk_rope_norm_store: unknown rotation style %d", style);
+    TQK_REQUIRE(rot_dim >= 0 && rot_dim % 2 == 0 && rot_dim <= key_dim, "tqk_rope_norm_store: rot_dim %d must be even and <= key_dim %d", rot_dim, key_dim);
+    TQK_REQUIRE(rot_dim == 0 || style == 0 || (cos_table && sin_table && max_positions > 0), "tqk_rope_norm_store: rotation without tables");
+    TQK_REQUIRE(!write_kv || (tok_seq && page_table && keys && values && table_width > 0), "tqk_rope_norm_store: no cache to write to");
+    if (n_tokens == 0) return 0;
+    hipStream_t s = (hipStream_t)stream;
+    dim3 grid(n_tokens, (n_heads + 2 * n_kv_heads + AM_WAVES - 1) / AM_WAVES);
+#define TQK_RNS(TA, TB) \
+    rope_norm_store_kernel<TA, TB><<<grid, AM_WAVES * TQK_WAVE, 0, s>>>((const TA*)qkv, (const TB*)bias, cos_table, sin_table, rot_dim, style, max_positions, \
+        normed, eps, tok_seq, tok_pos, page_table, table_width, (TA*)keys, (TA*)values, (TA*)q_out, n_heads, n_kv_heads, key_dim, value_dim, write_kv)
+    if (act_dtype == TQK_F32 && (!bias || bias_dtype == TQK_F32)) TQK_RNS(float, float);
+    else if (act_dtype == TQK_F32 && bias_dtype == TQK_BF16) TQK_RNS(float, bf16_t);
+    else if (act_dtype == TQK_BF16 && (!bias || bias_dtype == TQK_BF16)) TQK_RNS(bf16_t, bf16_t);
+    else if (act_dtype == TQK_BF16 && bias_dtype == TQK_F32) TQK_RNS(bf16_t, float);
+    else return tqk_fail("tqk_rope_norm_store: unknown dtypes %d, %d", act_dtype, bias_dtype);
+#undef TQK_RNS
+    return tqk_check_launch("tqk_rope_norm_store");
 }
 
 extern "C" int tqk_attention_masked_max_dim(void) { return AM_MAX_D; }

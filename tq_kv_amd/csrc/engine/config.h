@@ -30,5 +30,6 @@ std::vector<int32_t> tokenizer_stop_ids(const std::string& model_dir);
 void register_qwen2();
 void register_nikasun();
 void register_sizudra();
+void register_piditar();
 
 }  // namespace tq

@@ -78,6 +78,17 @@ TQ_KERNEL(unary_act, cptr, void*, int, long long, int, float, float, void*);
 TQ_KERNEL(row_gate, cptr, int, cptr, int, float*, int, int, void*);
 TQ_KERNEL(normed_rope_store, cptr, int, cptr, cptr, int, float, cf32, cf32, int, int, cptr, cptr, void*, ci32, ci32, ci32, int, void*, void*, void*,
           int, int, int, int, int, int, void*);
+TQ_KERNEL(rope_norm_store, cptr, int, cptr, int, cf32, cf32, int, int, int, int, float, ci32, ci32, ci32, int, void*, void*, void*, int, int, int, int,
+          int, int, void*);
+TQ_QUERY(int, conv_max_taps);
+TQ_QUERY(int, ssm_max_state);
+TQ_KERNEL(conv_state, cptr, int, long long, cf32, cf32, cf32, int, int, cf32, long long, ci32, ci32, ci32, ci32, float*, int, int, void*);
+TQ_KERNEL(conv_state_update, cptr, int, long long, cf32, int, float*, long long, ci32, ci32, ci32, int, int, void*);
+TQ_KERNEL(rglru_gates, cf32, cf32, cf32, cf32, cf32, cf32, float*, float*, int, int, int, void*);
+TQ_KERNEL(linear_scan, cf32, cf32, cptr, int, long long, cf32, float*, long long, ci32, ci32, ci32, void*, int, int, void*);
+TQ_KERNEL(ssm_scan, cf32, long long, cptr, int, long long, cf32, cf32, cf32, float*, long long, ci32, ci32, ci32, float*, int, int, int, int, int, void*);
+TQ_KERNEL(gated_part_norm, cf32, cptr, int, long long, cf32, float, void*, int, int, int, void*);
+TQ_KERNEL(add_rows, float*, cf32, long long, void*);
 TQ_QUERY(int, attention_masked_max_dim);
 TQ_QUERY(int, attention_masked_mfma_supported, int, int);
 TQ_QUERY(int, attention_masked_mfma_tile, int, int, int, int, int);

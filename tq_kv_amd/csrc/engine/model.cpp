@@ -164,8 +164,21 @@ Tensor Model::forward(StepContext& c, const CacheStore& cache, float* out) {
         stream.invalidate();            // what the gather prepared for the first norm is of the stream before this
         stream.copy_valid = copied;
     }
+    // Runs that take the embedding's output in again (a span of layers run several times, each pass fed the input anew) get it from a
+    // copy that lives for the whole step.
+    Tensor embedded;
+    for (const Run& run : s.order)
+        if (run.add_embedding && !embedded.defined()) {
+            embedded = Tensor(c.ws->alloc_for_step(h.bytes()), F32, {c.n_tokens, s.hidden_size});
+            copy_on_device(embedded.data, h.data, h.bytes(), c.stream);
+        }
     Stream* cur = &stream;
     for (size_t i = 0; i < s.order.size(); ++i) {
+        if (s.order[i].add_embedding) {
+            // (an update that is still pending is added by the next norm's kernel as always: the sum does not mind the order)
+            K::add_rows((float*)cur->h.data, (const float*)embedded.data, (long long)cur->h.numel(), c.stream);
+            cur->invalidate();
+        }
         // The layers take their temporaries from two arenas in turn.  What a layer leaves for the next one (an update
         // of the stream that is still pending) is read by that next layer, so the arena of the layer before the last
         // holds nothing that is still needed: unless a block handed on what it was given, which is looked for.

@@ -230,5 +230,6 @@ void register_builtin_parts();          // idempotent
 void register_latent_parts();           // parts_latent.cpp; called by register_builtin_parts
 void register_moe_parts();              // parts_moe.cpp; likewise
 void register_stream_parts();           // parts_stream.cpp; likewise
+void register_recurrent_parts();        // parts_recurrent.cpp; likewise
 
 }  // namespace tq

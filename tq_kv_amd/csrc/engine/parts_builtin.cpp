@@ -234,7 +234,8 @@ public:
 //
 // What other designs put around the same attention, all off unless given: value_dim (a head's values are of another
 // size than its keys); qk_norm with eps (every query and key head is divided by its root mean square and multiplied
-// by a weight of head_dim values, before the rotation); cap (scores become cap tanh(s / cap)); keep_first (with a
+// by a weight of head_dim values, before the rotation; with qk_norm_weight false and qk_norm_after_rotation true the heads are divided by
+// their root mean square after the rotation and there is no weight: then the projections may have biases and the rotation may go by pairs); cap (scores become cap tanh(s / cap)); keep_first (with a
 // window: a sequence's first positions stay visible, at their true places); sink (a learned number per head whose
 // exponential joins the softmax's denominator, with no key and no value); value_mix "source" (the values of the
 // step's tokens are handed to later layers) or "mixed" (v <- (1 - lambda) v + lambda v_source with a learned scalar,
@@ -265,6 +266,8 @@ public:
         prompt_tile_ = r.has("prompt_tile") ? (int)r.integer("prompt_tile") : 0;
         value_dim_ = r.has("value_dim") ? (int)r.integer("value_dim", 1) : head_dim_;
         qk_norm_ = r.boolean_or("qk_norm", false);
+        qk_norm_weight_ = r.boolean_or("qk_norm_weight", true);
+        norm_after_rotation_ = r.boolean_or("qk_norm_after_rotation", false);
         eps_ = qk_norm_ ? (float)r.number("eps") : 0.f;
         cap_ = r.has("cap") ? (float)r.number("cap", true) : 0.f;
         keep_first_ = (int)r.integer_or("keep_first", 0, 0);
@@ -278,13 +281,19 @@ public:
         mix_key_ = "attention." + r.string_or("value_mix_key", "values");
         if (keep_first_ > 0 && window_ == 0) raise(TQE_ERR_ARGUMENT, "attention: keep_first %d without a window", keep_first_);
         extras_ = value_dim_ != head_dim_ || qk_norm_ || cap_ > 0.f || keep_first_ > 0 || has_sink_ || value_mix_ != MIX_NONE;
-        if (extras_ && (qkv_bias_ || out_bias_)) raise(TQE_ERR_ARGUMENT, "attention: biases go with none of value_dim, qk_norm, cap, keep_first, sink, value_mix");
+        if (qk_norm_ && qk_norm_weight_ == norm_after_rotation_)
+            raise(TQE_ERR_ARGUMENT, "attention: the heads' norm is either weighted and in front of the rotation, or without a weight and after it");
+        // the kernel that adds biases, turns and then norms without a weight stands for every such combination but mixed values
+        const bool turned_ok = extras_ && (!qk_norm_ || norm_after_rotation_) && value_mix_ == MIX_NONE;
+        if (extras_ && (out_bias_ || (qkv_bias_ && !turned_ok)))
+            raise(TQE_ERR_ARGUMENT, "attention: with value_dim, cap, keep_first or sink the projections may have biases where the heads' norm has no weight and values are not mixed; the output has none");
         {
             const Json& names = spec.params["names"];
             auto name = [&](const char* role, const char* fallback) { return names[role].is_string() ? names[role].as_string() : std::string(fallback); };
             n_q_ = name("q", "q_proj.weight"); n_k_ = name("k", "k_proj.weight"); n_v_ = name("v", "v_proj.weight"); n_o_ = name("o", "o_proj.weight");
             n_q_norm_ = name("q_norm", "q_norm.weight"); n_k_norm_ = name("k_norm", "k_norm.weight");
             n_sink_ = name("sink", "sink"); n_mix_ = name("mix", "value_mix");
+            n_qb_ = name("q_bias", "q_proj.bias"); n_kb_ = name("k_bias", "k_proj.bias"); n_vb_ = name("v_bias", "v_proj.bias");
         }
         if (r.has("prompt_tile") && prompt_tile_ != 16 && prompt_tile_ != 32 && prompt_tile_ != 64 && prompt_tile_ != 128)
             raise(TQE_ERR_ARGUMENT, "attention: prompt_tile must be 16, 32, 64 or 128, got %d", prompt_tile_);
@@ -306,8 +315,9 @@ public:
         takes_rows = true;
         if (extras_) {
             const Position::Tables tb = position_->tables();
-            if (position_->has_apply() || (tb.style != STYLE_NONE && (tb.style != STYLE_HALVES || tb.rot_dim > head_dim_)))
-                raise(TQE_ERR_ARGUMENT, "attention: with value_dim, qk_norm, cap, keep_first, sink or value_mix the position part must turn in halves from tables");
+            turned_first_ = turned_ok && (qkv_bias_ || norm_after_rotation_ || tb.style == STYLE_PAIRS);
+            if (position_->has_apply() || tb.rot_dim > head_dim_ || (tb.style != STYLE_NONE && tb.style != STYLE_HALVES && !turned_ok))
+                raise(TQE_ERR_ARGUMENT, "attention: with value_dim, qk_norm, cap, keep_first, sink or value_mix the position part must turn from tables (in halves where the heads' norm has a weight or values are mixed)");
         }
     }
 
@@ -317,7 +327,7 @@ public:
         auto b = [](int64_t a) { TensorSpec t; t.shape = {a}; return t; };
         TensorSpecs t = {{n_q_, w(q, hidden_)}, {n_k_, w(kv, hidden_)}, {n_v_, w((int64_t)n_kv_heads_ * value_dim_, hidden_)},
                          {n_o_, w(hidden_, (int64_t)n_heads_ * value_dim_)}};
-        if (qk_norm_) {
+        if (qk_norm_ && qk_norm_weight_) {
             TensorSpec n = b(head_dim_);
             n.init = "one_plus_normal";
             n.std_dev = 0.1;
@@ -327,7 +337,7 @@ public:
         if (has_sink_) { TensorSpec s = b(n_heads_); s.std_dev = 1.0; t.push_back({n_sink_, s}); }
         // the source layer of a mix has the scalar too, and does not use it
         if (value_mix_ != MIX_NONE) { TensorSpec s; s.shape = {}; s.std_dev = 0.3; t.push_back({n_mix_, s}); }
-        if (qkv_bias_) { t.push_back({"q_proj.bias", b(q)}); t.push_back({"k_proj.bias", b(kv)}); t.push_back({"v_proj.bias", b(kv)}); }
+        if (qkv_bias_) { t.push_back({n_qb_, b(q)}); t.push_back({n_kb_, b(kv)}); t.push_back({n_vb_, b((int64_t)n_kv_heads_ * value_dim_)}); }
         if (out_bias_) t.push_back({"o_proj.bias", b(hidden_)});
         return t;
     }
@@ -336,10 +346,10 @@ public:
 
     void load(Loaded& t, hipStream_t stream) override {
         OwnedPtr qkv = stacked({take(t, n_q_.c_str()), take(t, n_k_.c_str()), take(t, n_v_.c_str())}, stream);
-        if (qk_norm_) { q_norm_ = take(t, n_q_norm_.c_str()); k_norm_ = take(t, n_k_norm_.c_str()); }
+        if (qk_norm_ && qk_norm_weight_) { q_norm_ = take(t, n_q_norm_.c_str()); k_norm_ = take(t, n_k_norm_.c_str()); }
         if (has_sink_) sink_ = take(t, n_sink_.c_str());
         if (value_mix_ != MIX_NONE) mix_ = take(t, n_mix_.c_str());
-        if (qkv_bias_) b_qkv_ = stacked({take(t, "q_proj.bias"), take(t, "k_proj.bias"), take(t, "v_proj.bias")}, stream);
+        if (qkv_bias_) b_qkv_ = stacked({take(t, n_qb_.c_str()), take(t, n_kb_.c_str()), take(t, n_vb_.c_str())}, stream);
         if (out_bias_) b_o_ = take(t, "o_proj.bias");
         w_qkv_ = make_weight(qkv, 1, false, stream);
         w_o_ = make_weight(take(t, n_o_.c_str()), 1, b_o_ != nullptr, stream);
@@ -350,8 +360,8 @@ public:
         if (name == "qkv.bias") return b_qkv_;
         if (name == "o_proj.weight") return w_o_.rows;
         if (name == "o_proj.weight.packed") return w_o_.packed;
-        if (qk_norm_ && name == n_q_norm_) return q_norm_;
-        if (qk_norm_ && name == n_k_norm_) return k_norm_;
+        if (q_norm_ && name == n_q_norm_) return q_norm_;
+        if (k_norm_ && name == n_k_norm_) return k_norm_;
         if (has_sink_ && name == n_sink_) return sink_;
         if (value_mix_ != MIX_NONE && name == n_mix_) return mix_;
         return nullptr;
@@ -397,7 +407,8 @@ public:
         const int n_pages = (int)entry.keys.shape[0];
         if (extras_) {
             if (x.lazy) raise(TQE_ERR_STATE, "attention: this configuration takes no folded norm");
-            normed_qkv(c, x.x, entry, table, q);
+            if (turned_first_) turned_qkv(c, x.x, entry, table, q);
+            else normed_qkv(c, x.x, entry, table, q);
         } else if (x.lazy || (c.fuse_small && entry.writes && fused_qkv_ok(c))) {
             if (x.lazy && !entry.writes) raise(TQE_ERR_STATE, "a run that reads another run's cache cannot take a folded norm");
             const Position::Tables tb = position_->tables();
@@ -459,6 +470,20 @@ private:
                              turn ? (int)tb.cos.shape[0] : 0, mix_ ? mix_->t.data : nullptr, mix_with, mix_keep, c.dev.tok_seq, c.dev.tok_pos,
                              write ? table.dev : nullptr, write ? table.width : 0, write ? entry.keys.data : nullptr, write ? entry.values.data : nullptr,
                              q.data, (int)n, n_heads_, n_kv_heads_, head_dim_, value_dim_, write ? 1 : 0, c.stream);
+    }
+
+    // product, then biases, rotation (halves or pairs), the heads' norm without a weight after it, and the cache write in one kernel
+    void turned_qkv(StepContext& c, const Tensor& x, const CacheEntry& entry, const StepContext::Table& table, Tensor& q) {
+        const int64_t n = x.shape[0];
+        Product p = linear(c, x, w_qkv_, nullptr, x.dtype);
+        const Position::Tables tb = position_->tables();
+        const bool turn = tb.style != STYLE_NONE;
+        const bool write = entry.writes;
+        K::rope_norm_store(p.t.data, p.t.dtype, b_qkv_ ? b_qkv_->t.data : nullptr, b_qkv_ ? b_qkv_->t.dtype : 0, turn ? (const float*)tb.cos.data : nullptr,
+                           turn ? (const float*)tb.sin.data : nullptr, turn ? tb.rot_dim : 0, turn ? tb.style : 0, turn ? (int)tb.cos.shape[0] : 0,
+                           qk_norm_ ? 1 : 0, eps_, c.dev.tok_seq, c.dev.tok_pos, write ? table.dev : nullptr, write ? table.width : 0,
+                           write ? entry.keys.data : nullptr, write ? entry.values.data : nullptr, q.data, (int)n, n_heads_, n_kv_heads_, head_dim_, value_dim_,
+                           write ? 1 : 0, c.stream);
     }
 
     // Attention of rows (sequence tok_seq[r], position tok_pos[r]) with the cap, the kept first positions and the sink.  bfloat16 on the
@@ -646,8 +671,9 @@ private:
     enum { MIX_NONE = 0, MIX_SOURCE = 1, MIX_MIXED = 2 };
     int value_dim_, keep_first_, value_mix_ = MIX_NONE;
     bool qk_norm_ = false, has_sink_ = false, extras_ = false, cache_keeps_all_ = false;
+    bool qk_norm_weight_ = true, norm_after_rotation_ = false, turned_first_ = false;
     float eps_ = 0.f, cap_ = 0.f;
-    std::string mix_key_, n_q_, n_k_, n_v_, n_o_, n_q_norm_, n_k_norm_, n_sink_, n_mix_;
+    std::string mix_key_, n_q_, n_k_, n_v_, n_o_, n_q_norm_, n_k_norm_, n_sink_, n_mix_, n_qb_, n_kb_, n_vb_;
     std::shared_ptr<Position> position_;
     Weight w_qkv_, w_o_;
     OwnedPtr b_qkv_, b_o_, q_norm_, k_norm_, sink_, mix_;
@@ -902,6 +928,7 @@ void register_builtin_parts() {
         register_latent_parts();
         register_moe_parts();
         register_stream_parts();
+        register_recurrent_parts();
         register_kind("block", "pre_norm", [](const PartSpec& s, BuildEnv& e) { return std::make_shared<PreNormBlock>(s, e); });
     });
 }

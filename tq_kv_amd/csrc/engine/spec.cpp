@@ -118,6 +118,7 @@ Json ModelSpec::to_json() const {
         Json o = Json::object();
         o.set("layer", r.layer);
         o.set("cache_of", r.cache_of >= 0 ? Json(r.cache_of) : Json());
+        if (r.add_embedding) o.set("add_embedding", true);
         rs.push(o);
     }
     j.set("order", rs);
@@ -159,6 +160,7 @@ ModelSpec ModelSpec::from_json(const Json& j) {
         run.layer = (int)o["layer"].as_int();
         run.cache_of = o["cache_of"].is_int() ? (int)o["cache_of"].as_int() : -1;
         if (o["cache_of"].is_int() && run.cache_of < 0) run.cache_of = INT32_MIN;        // named, and wrong: refused by the model
+        run.add_embedding = o["add_embedding"].is_bool() && o["add_embedding"].as_bool();
         s.order.push_back(run);
     }
     s.final_norm = PartSpec::from_json(j["final_norm"], "final norm");

@@ -66,9 +66,11 @@ struct LayerSpec {
 
 // One entry of the run order: run layer `layer`; cache_of >= 0 names an earlier entry whose
 // cache this run reads instead of keeping its own.
+// add_embedding: the embedding's output (the stream as it was before the first run) is added to the stream before this run.
 struct Run {
     int layer = 0;
     int cache_of = -1;
+    bool add_embedding = false;
 };
 
 struct ModelSpec {

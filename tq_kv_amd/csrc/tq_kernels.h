@@ -312,6 +312,50 @@ int tqk_attention_masked_mfma(const void* q, const void* keys, const void* value
                               int tile_queries, int n_rows, int n_parts, void* part_out, void* part_ml, void* out, int n_heads, int n_kv_heads,
                               int key_dim, int value_dim, void* stream);
 
+/* Bias, rotation, then a norm without a weight (attention_masked.hip): rows of qkv are [heads * key_dim | kv heads * key_dim | kv heads *
+ * value_dim]; bias (optional) has a row's layout; q and k are turned (style 1: in halves, 2: element 2i with 2i + 1, 0: not at all) and then,
+ * if normed, every head is divided by its root mean square (eps inside the root).  q goes to q_out, keys and values into the pages. */
+int tqk_rope_norm_store(const void* qkv, int act_dtype, const void* bias, int bias_dtype, const float* cos_table, const float* sin_table,
+                        int rot_dim, int style, int max_positions, int normed, float eps, const int32_t* tok_seq, const int32_t* tok_pos,
+                        const int32_t* page_table, int table_width, void* keys, void* values, void* q_out, int n_tokens, int n_heads,
+                        int n_kv_heads, int key_dim, int value_dim, int write_kv, void* stream);
+
+/* Mixers with a fixed-size state (recurrent.hip).  A step is a packed batch: token t belongs to sequence tok_seq[t] of the step at position
+ * tok_pos[t]; sequence s brings seq_new[s] tokens from packed row cu[s] on, had seq_start[s] positions before, and its state is row seq_slot[s]
+ * (rows state_stride floats apart).  Small parameters are float32.
+ *
+ * tqk_conv_state: out[t, c] = act(bias[c] + sum_k w[c, k] in(t - (taps - 1 - k), c)), in = x + in_bias for the step's rows (x: rows x_stride
+ * values apart, any float dtype) and the state's [taps - 1][channels] (oldest first) for what came before; activation 0: none, 1: silu.
+ * tqk_conv_state_update: the state after the step (call it after every reader of the old one). */
+#define TQK_CONV_MAX_TAPS 8
+int tqk_conv_max_taps(void);
+int tqk_conv_state(const void* x, int x_dtype, long long x_stride, const float* in_bias, const float* w, const float* bias, int taps,
+                   int activation, const float* state, long long state_stride, const int32_t* tok_seq, const int32_t* tok_pos,
+                   const int32_t* seq_slot, const int32_t* seq_start, float* out, int n_tokens, int channels, void* stream);
+int tqk_conv_state_update(const void* x, int x_dtype, long long x_stride, const float* in_bias, int taps, float* state, long long state_stride,
+                          const int32_t* cu, const int32_t* seq_new, const int32_t* seq_slot, int n_seqs, int channels, void* stream);
+/* Gates of a real-gated linear recurrent unit: r = sigmoid(Wa u + ba), i = sigmoid(Wi u + bi) with block-diagonal Wa, Wi given as
+ * [blocks][in][out]; a = exp(decay_c r) (decay_c = -8 softplus(lam), per channel); g = sqrt(1 - a^2) i u. */
+int tqk_rglru_gates(const float* u, const float* wa_t, const float* wi_t, const float* ba, const float* bi, const float* decay_c, float* a_out,
+                    float* g_out, int n_tokens, int width, int blocks, void* stream);
+/* S_t = a_t S_(t-1) + g_t per sequence and channel from the state (one float a channel), which is left at the last S;
+ * out_t = S_t gelu_tanh(y_t + y_bias) in the activation dtype. */
+int tqk_linear_scan(const float* a, const float* g, const void* y, int act_dtype, long long y_stride, const float* y_bias, float* state,
+                    long long state_stride, const int32_t* cu, const int32_t* seq_new, const int32_t* seq_slot, void* out, int n_seqs,
+                    int width, void* stream);
+/* The selective state-space recurrence with one decay per head: xbc rows are [x: heads * p_dim | B: groups * n_state | C: groups * n_state];
+ * dt = softplus(dt_raw[t, h] + dt_bias[h]); S_t = exp(-exp(a_log[h]) dt) S_(t-1) + dt B_t x_t^T; y_t = S_t^T C_t + d_skip[h] x_t.
+ * The state of a slot: [heads][n_state][p_dim] float32. */
+int tqk_ssm_max_state(void);
+int tqk_ssm_scan(const float* xbc, long long xbc_stride, const void* dt_raw, int dt_dtype, long long dt_stride, const float* dt_bias,
+                 const float* a_log, const float* d_skip, float* state, long long state_stride, const int32_t* cu, const int32_t* seq_new,
+                 const int32_t* seq_slot, float* y_out, int n_seqs, int heads, int groups, int n_state, int p_dim, void* stream);
+/* out = norm_parts(y silu(z)) w: `parts` equal parts of a row, each divided by its own root mean square. */
+int tqk_gated_part_norm(const float* y, const void* z, int act_dtype, long long z_stride, const float* w, float eps, void* out, int n_tokens,
+                        int size, int parts, void* stream);
+/* h[i] += x[i], float32 */
+int tqk_add_rows(float* h, const float* x, long long n, void* stream);
+
 /* out[r] = lowest index of the largest value of logits[r, :]; scratch: at least
  * tqk_argmax_scratch_floats(n_rows, vocab) floats of device memory. */
 int tqk_argmax_scratch_floats(int n_rows, int vocab);

@@ -133,9 +133,11 @@ class LayerSpec:
 @dataclass(frozen=True)
 class Run:
     """One entry of the run order: run layer `layer`.  `cache_of` names an earlier
-    entry of the order whose cache this run reads instead of keeping its own."""
+    entry of the order whose cache this run reads instead of keeping its own.
+    `add_embedding`: the embedding's output is added to the stream before this run."""
     layer: int
     cache_of: Optional[int] = None
+    add_embedding: bool = False
 
 
 @dataclass(frozen=True)
@@ -164,7 +166,8 @@ class ModelSpec:
             "architecture": self.architecture, "vocab_size": int(self.vocab_size), "hidden_size": int(self.hidden_size),
             "max_positions": int(self.max_positions), "embedding_name": self.embedding_name,
             "layers": [{"prefix": l.prefix, "block": l.block.to_json()} for l in self.layers],
-            "order": [{"layer": int(r.layer), "cache_of": None if r.cache_of is None else int(r.cache_of)} for r in self.order],
+            "order": [dict({"layer": int(r.layer), "cache_of": None if r.cache_of is None else int(r.cache_of)},
+                            **({"add_embedding": True} if r.add_embedding else {})) for r in self.order],
             "final_norm": self.final_norm.to_json(), "final_norm_prefix": self.final_norm_prefix, "head_name": self.head_name,
             "eos_token_ids": [int(t) for t in self.eos_token_ids], "embedding_scale": self.embedding_scale,
             "stream_position": None if self.stream_position is None else self.stream_position.to_json(),
@@ -177,7 +180,7 @@ class ModelSpec:
             architecture=j["architecture"], vocab_size=j["vocab_size"], hidden_size=j["hidden_size"], max_positions=j["max_positions"],
             embedding_name=j["embedding_name"],
             layers=[LayerSpec(l["prefix"], PartSpec.from_json(l["block"])) for l in j["layers"]],
-            order=[Run(r["layer"], r.get("cache_of")) for r in j["order"]],
+            order=[Run(r["layer"], r.get("cache_of"), bool(r.get("add_embedding", False))) for r in j["order"]],
             final_norm=PartSpec.from_json(j["final_norm"]), final_norm_prefix=j["final_norm_prefix"], head_name=j.get("head_name"),
             eos_token_ids=tuple(j.get("eos_token_ids") or ()), embedding_scale=j.get("embedding_scale"),
             stream_position=None if j.get("stream_position") is None else PartSpec.from_json(j["stream_position"]),
