@@ -94,7 +94,7 @@ public:
                 {n_decay_, vector_of(width_, 1.0)}, {n_o_, matrix(hidden_, width_)}};
     }
     void load(Loaded& t, hipStream_t stream) override {
-        w_yx_ = make_weight(stack_rows({take(t, n_y_), take(t, n_x_)}, stream), 2, false, stream);
+        w_yx_ = make_weight(stack_rows({take(t, n_y_), take(t, n_x_)}, stream), 1, false, stream);
         w_o_ = make_weight(take(t, n_o_), 1, false, stream);
         y_bias_ = as_floats(take(t, n_yb_), stream);
         x_bias_ = as_floats(take(t, n_xb_), stream);
