@@ -59,9 +59,11 @@ def config_single(kind, width=64):
     return config(97, width, [(mix, 48)], scale=5.0)
 
 
-def weights(cfg, seed, store=torch.bfloat16, forgetful=False):
-    """name -> tensor of the store dtype.  Products keep the size of what they read (std 1/sqrt(inputs)).  forgetful: the
-    recurrences' decays are driven to zero, so that a token's output depends on the convolution's reach alone."""
+def weights(cfg, seed, store=torch.bfloat16, memory="some"):
+    """name -> tensor of the store dtype.  Products keep the size of what they read (std 1/sqrt(inputs)).  memory "none": the
+    recurrences' decays are driven to zero, so that a token's output depends on the convolution's reach alone; "long": decays
+    close to one, so that the state holds a token for hundreds of positions."""
+    forgetful, lasting = memory == "none", memory == "long"
     g = torch.Generator().manual_seed(seed)
 
     def lin(o, i, gain=1.0):
@@ -93,7 +95,9 @@ def weights(cfg, seed, store=torch.bfloat16, forgetful=False):
             for n in ("ra", "ri"):
                 w[q + n] = (torch.randn(nb, bs, bs, generator=g) / math.sqrt(bs)).to(store)
                 w[q + n + ".b"] = (0.5 * torch.randn(nb, bs, generator=g)).to(store)
-            w[q + "lam"] = vec(W, 40.0 if forgetful else -2.0, 1.0)
+            if forgetful:
+                w[q + "ra.b"] = w[q + "ra.b"] + 12.0            # r is 1 but for rounding, whatever the input
+            w[q + "lam"] = vec(W, 40.0 if forgetful else -6.0 if lasting else -2.0, 1.0 if not lasting else 0.3)
             w[q + "o"] = lin(D, W)
         else:
             H, P, N, G = m["heads"], m["vdim"], m["state"], m["groups"]
@@ -101,8 +105,8 @@ def weights(cfg, seed, store=torch.bfloat16, forgetful=False):
             w[q + "in"] = lin(2 * inner + 2 * G * N + H, D)
             w[q + "conv"] = (torch.randn(ch, m["conv"], generator=g) * 0.5).to(store)
             w[q + "conv.b"] = vec(ch, 0.0, 0.2)
-            w[q + "dt_bias"] = vec(H, 30.0 if forgetful else -1.0, 0.5)
-            w[q + "A_log"] = vec(H, 2.0 if forgetful else -0.5, 0.5)
+            w[q + "dt_bias"] = vec(H, 30.0 if forgetful else -3.0 if lasting else -1.0, 0.5)
+            w[q + "A_log"] = vec(H, 2.0 if forgetful else -2.0 if lasting else -0.5, 0.5)
             w[q + "D"] = vec(H, 1.0, 0.3)
             w[q + "norm"] = vec(inner, 1.0, 0.1)
             w[q + "o"] = lin(D, inner)

@@ -130,18 +130,18 @@ MAKERS = {"mixed": C.config_mixed, "ones": C.config_ones, "odd": C.config_odd, "
           "rglru": lambda: C.config_single("rglru"), "mamba2": lambda: C.config_single("mamba2")}
 
 
-def model(name, tmp_path_factory, forgetful=False):
-    key = (name, forgetful)
+def model(name, tmp_path_factory, memory="some"):
+    key = (name, memory)
     if key not in _MODELS:
         cfg = MAKERS[name]()
-        w = C.weights(cfg, seed=11 + len(name), forgetful=forgetful)
+        w = C.weights(cfg, seed=11 + len(name), memory=memory)
         folder = C.write_folder(str(tmp_path_factory.mktemp("piditar_%s" % name)), cfg, w)
         _MODELS[key] = (cfg, w, folder, {})
     return _MODELS[key]
 
 
-def engine(name, dtype, tmp_path_factory, forgetful=False, max_tokens=4096, slots=8):
-    cfg, w, folder, engines = model(name, tmp_path_factory, forgetful)
+def engine(name, dtype, tmp_path_factory, memory="some", max_tokens=4096, slots=8):
+    cfg, w, folder, engines = model(name, tmp_path_factory, memory)
     if dtype not in engines:
         engines[dtype] = Engine(Model.from_dir(folder, dtype=dtype), max_tokens=max_tokens, max_slots=slots)
     return cfg, w, engines[dtype]
@@ -265,22 +265,19 @@ def test_a_token_reaches_every_later_position_through_attention_and_none_before(
 
 
 def test_one_key_far_away_among_hundreds_carries_the_output(tmp_path_factory):
-    """The keys of one token are made to point where a late query points, many times longer than any other: the output at the query is that
-    token's value, wherever the token stands (first, at a page's border, far back) and however the query comes (prompt or decoded)."""
-    cfg = C.config(60, 32, [(C.attention(2, 1, 16, 24, 0, scale=4.0, softcap=60.0), None)], scale=1.0)
-    w = C.weights(cfg, 4)
+    """Two tokens have an element of the embedding to themselves; the keys of the one and the queries of the other read it with one and the
+    same long vector, so that this key's score stands far above three hundred random ones: the output at the query is that token's value,
+    wherever the token stands (first, at a page's border, far back) and however the query comes (in the prompt or decoded)."""
+    cfg = C.config(60, 32, [(C.attention(2, 1, 64, 24, 0, scale=1.0, softcap=100.0), None)], scale=1.0)
     n, special, asker = 330, 7, 11
     toks = [t if t not in (special, asker) else 20 for t in C.tokens(n, cfg["vocab"], 2)]
-    f = C.as_float(w)
-    # without rotation the query of `asker` and the key of `special` are made equal directions; every other key is random
-    for name in ("l0.mix.q", "l0.mix.k"):
-        f[name] = f[name] * 0.05
-    f["l0.mix.q.b"] = torch.zeros_like(f["l0.mix.q.b"])
-    f["l0.mix.k.b"] = torch.zeros_like(f["l0.mix.k.b"])
-    e = torch.nn.functional.normalize(f["embed"], dim=-1)
-    direction = torch.randn(16)
-    f["l0.mix.k"] = f["l0.mix.k"] + torch.outer(direction, e[special]) * 3.0
-    f["l0.mix.q"] = f["l0.mix.q"] + torch.outer(direction.repeat(2), e[asker]) * 3.0
+    f = C.as_float(C.weights(cfg, 4))
+    f["embed"][:, 0] = 0.0
+    f["embed"][special, 0] = f["embed"][asker, 0] = 3.0
+    direction = torch.randn(64)
+    f["l0.mix.k"][:, 0] = 3.0 * direction
+    f["l0.mix.q"][:, 0] = 3.0 * direction.repeat(2)
+    f["l0.mix.v"] = f["l0.mix.v"] * 3.0
     w = {k: v.to(torch.bfloat16) for k, v in f.items()}
     folder = C.write_folder(str(tmp_path_factory.mktemp("piditar_far")), cfg, w)
     for dtype in DTYPES:
@@ -301,13 +298,15 @@ def test_one_key_far_away_among_hundreds_carries_the_output(tmp_path_factory):
 def test_a_forgetful_recurrence_sees_exactly_the_convolutions_reach(kind, dtype, tmp_path_factory):
     """One recurrent layer whose decay is driven to zero: the state forgets everything at once, and what is left is the short convolution.
     Changing the token at j changes the logits at i if and only if i - taps < j <= i; in prompts, across portions' borders, and decoded."""
-    cfg, w, eng = engine(kind, dtype, tmp_path_factory, forgetful=True)
+    cfg, w, eng = engine(kind, dtype, tmp_path_factory, memory="none")
     taps = cfg["layers"][0]["mixer"]["conv"]
     n = 140
     toks = C.tokens(n, cfg["vocab"], 9)
     for how in ("prompt", "portions", "decoded"):
         base = logits_of(eng, toks, how, n)
-        C.close(base, C.plain_logits(cfg, w, toks), dtype, how)
+        # (with the state gone a position's output hangs on few numbers, and bfloat16 products move a row here and there by a fifth of
+        # the spread: bfloat16 is held to the plain implementation with its products rounded the same way)
+        C.close(base, C.plain_logits(cfg, w, toks, DT[dtype]), dtype, how)
         for i in (2, 62, 63, 64, 65, 101, 130, 131, 139):
             for back in (0, 1, taps - 1, taps, taps + 1, 60):
                 j = i - back
@@ -326,12 +325,12 @@ def test_a_forgetful_recurrence_sees_exactly_the_convolutions_reach(kind, dtype,
 @pytest.mark.parametrize("kind", ["rglru", "mamba2"])
 def test_a_recurrence_carries_the_first_token_to_the_last(kind, dtype, tmp_path_factory):
     """With decays near one the state remembers: the first token moves the logits hundreds of positions on, decoded or not."""
-    cfg, w, eng = engine(kind, dtype, tmp_path_factory)
+    cfg, w, eng = engine(kind, dtype, tmp_path_factory, memory="long")
     n = 260
     toks = C.tokens(n, cfg["vocab"], 10)
     changed = [(toks[0] + 1) % cfg["vocab"]] + toks[1:]
     want, want_changed = C.plain_logits(cfg, w, toks), C.plain_logits(cfg, w, changed)
-    assert C.row_errors(want_changed[-1:], want[-1:]).item() > 1e-3
+    assert C.row_errors(want_changed[-1:], want[-1:]).item() > 2e-3          # ten times what float32 is held to
     for cuts in ([], [200] + list(range(201, n))):
         C.close(run_cut(eng, toks, cuts), want, dtype, "cuts %s" % cuts[:2])
         C.close(run_cut(eng, changed, cuts), want_changed, dtype, "another first token, cuts %s" % cuts[:2])
