@@ -20,7 +20,9 @@ Nikasun design (attention through cached latents with a window, routed experts) 
 model's layers, beside a Qwen2 shape of the same width, depth, heads and active feed-forward size: prompt pass and
 decoding of both, tokens a second.  `python bench.py --masked` does the same for the Sizudra design (attention with normed
 heads, mixed values, and in every other layer a score cap, a window that keeps the first positions and a sink; a pair
-embedding; norms on the parts' outputs; routed experts without a gate product).
+embedding; norms on the parts' outputs; routed experts without a gate product).  `python bench.py --recurrent` does it for the
+Piditar design (layers of attention, of a real-gated linear recurrent unit and of a selective state-space mixer, each with a dense
+feed-forward).
 """
 import argparse
 import gc
@@ -49,6 +51,7 @@ def main():
     ap.add_argument("--latent", action="store_true", help="measure the Nikasun design beside a Qwen2 shape of equal size instead of the default workload")
     ap.add_argument("--latent-sizes", default="2048,4096", help="widths of the --latent and --masked comparisons")
     ap.add_argument("--masked", action="store_true", help="measure the Sizudra design beside a Qwen2 shape of equal size instead of the default workload")
+    ap.add_argument("--recurrent", action="store_true", help="measure the Piditar design beside a Qwen2 shape of equal size instead of the default workload")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this library runs on one GPU; --gpus %d is not supported" % args.gpus)
@@ -156,6 +159,9 @@ def main():
         return design_comparison("nikasun", latent_shapes, args, torch, Model, Engine, note, timed_prefill, decode, random_prompts, release)
     if args.masked:
         return design_comparison("sizudra", masked_shapes, args, torch, Model, Engine, note, timed_prefill, decode, random_prompts, release)
+
+    if args.recurrent:
+        return design_comparison("piditar", recurrent_shapes, args, torch, Model, Engine, note, timed_prefill, decode, random_prompts, release)
 
     # -- the headline shape -------------------------------------------------------------------------
     raw = dict(catalog.find(args.shape))
@@ -336,6 +342,26 @@ def masked_shapes(width, layers=4):
              "use_sliding_window": True, "sliding_window": 1024, "max_window_layers": layers // 2}
     return sizudra, qwen2, {"width": width, "layers": layers, "heads": heads, "kv_heads": kv_heads, "experts": experts, "top": top, "expert_ff": ff,
                             "shared_ff": shared, "dense_ff": active, "window": 1024, "keep_first": 4}
+
+
+def recurrent_shapes(width, layers=4):
+    """A Piditar configuration (attention, recurrent unit, state-space mixer, recurrent unit) and a Qwen2 one of the same width, depth, heads,
+    head size and feed-forward size."""
+    heads, dim = width // 128, 128
+    kv_heads = max(1, heads // 4)
+    ff = 3 * width
+    attention = {"heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": dim, "scale": dim ** -0.5, "softcap": 50.0, "rot": {"base": 10000.0, "dims": 64}}
+    rglru = {"width": width, "blocks": heads, "conv": 4}
+    mamba2 = {"heads": 2 * width // 64, "vdim": 64, "state": 128, "groups": 1, "conv": 4, "norm_groups": 1}
+    kinds = [("attention", attention), ("rglru", rglru), ("mamba2", mamba2), ("rglru", rglru)]
+    lay = [{"type": kinds[l % 4][0], "mixer": kinds[l % 4][1], "mlp": {"kind": "dense", "ff": ff}} for l in range(layers)]
+    piditar = {"architecture": "Piditar", "vocab": 32000, "width": width, "embedding": {"scale": width ** 0.5}, "norm": {"eps": 1e-5}, "layers": lay,
+               "loop": {"start": 0, "stop": layers, "times": 1}, "max_positions": 8192}
+    qwen2 = {"architectures": ["Qwen2ForCausalLM"], "model_type": "qwen2", "hidden_act": "silu", "vocab_size": 32000, "hidden_size": width,
+             "intermediate_size": ff, "num_hidden_layers": layers, "num_attention_heads": heads, "num_key_value_heads": kv_heads,
+             "head_dim": dim, "rms_norm_eps": 1e-5, "rope_theta": 10000.0, "max_position_embeddings": 8192, "tie_word_embeddings": True}
+    return piditar, qwen2, {"width": width, "layers": layers, "heads": heads, "kv_heads": kv_heads, "ff": ff, "rglru_width": width, "rglru_blocks": heads,
+                            "mamba2_heads": mamba2["heads"], "mamba2_state": 128, "conv": 4}
 
 
 def design_comparison(design, shapes, args, torch, Model, Engine, note, timed_prefill, decode, random_prompts, release):
