@@ -60,7 +60,7 @@ def step_ctx(cache, items):
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("mix", MIXERS, ids=lambda m: m[0] + "-" + "x".join(str(v) for v in m[1].values() if isinstance(v, int)))
 def test_a_mixer_alone(dtype, mix):
-    """Two sequences in shared steps: one in portions of 100, 26, 2 and 2 tokens and then token by token, across a page's border; the other whole
+    """Two sequences in shared steps: one in portions of 230, 26, 2 and 2 tokens and then token by token, across pages' borders; the other whole
     beside the first portion.  Then the slots are given back and taken again: nothing of the first use may be left."""
     kind, m = mix
     hidden, eps = 88, 1e-5
@@ -73,9 +73,10 @@ def test_a_mixer_alone(dtype, mix):
     part.load({k: v.to(DT[dtype]).to(DEV) for k, v in w.items()})
     cache = Cache([part.cache_need()], [None], 64 * 8, 2, DT[dtype], DEV)
     assert (len(cache.state_groups) == 1) == (kind != "attention")
-    xs = [torch.randn(n, hidden).to(DT[dtype]) for n in (150, 40)]
+    xs = [torch.randn(n, hidden).to(DT[dtype]) for n in (300, 40)]
     want = [plain.mixer(kind, x.float(), C.as_float(w), "", m, eps, torch.arange(x.shape[0]), DT[dtype]) for x in xs]
-    plan = [[(0, 0, 100), (1, 0, 40)], [(0, 100, 126)], [(0, 126, 128)], [(0, 128, 130)]] + [[(0, t, t + 1)] for t in range(130, 150)]
+    # (the first step is long enough for the recurrences to run in chunks, beside a sequence shorter than a chunk; the second is not)
+    plan = [[(0, 0, 230), (1, 0, 40)], [(0, 230, 256)], [(0, 256, 258)], [(0, 258, 260)]] + [[(0, t, t + 1)] for t in range(260, 300)]
     for use in range(2):
         slots = [cache.acquire(), cache.acquire()]
         got = [[], []]

@@ -87,6 +87,10 @@ TQ_KERNEL(conv_state_update, cptr, int, long long, cf32, int, float*, long long,
 TQ_KERNEL(rglru_gates, cf32, cf32, cf32, cf32, cf32, cf32, float*, float*, int, int, int, void*);
 TQ_KERNEL(linear_scan, cf32, cf32, cptr, int, long long, cf32, float*, long long, ci32, ci32, ci32, void*, int, int, void*);
 TQ_KERNEL(ssm_scan, cf32, long long, cptr, int, long long, cf32, cf32, cf32, float*, long long, ci32, ci32, ci32, float*, int, int, int, int, int, void*);
+TQ_KERNEL(linear_chunks, cf32, cf32, cptr, int, long long, cf32, ci32, ci32, int, float*, float*, void*, int, int, void*);
+TQ_KERNEL(chunk_carry, cf32, long long, int, float*, ci32, ci32, float*, long long, int, long long, void*);
+TQ_KERNEL(ssm_steps, cptr, int, long long, cf32, cf32, float*, float*, int, int, void*);
+TQ_KERNEL(ssm_chunks, cf32, long long, cf32, cf32, cf32, ci32, ci32, int, float*, float*, float*, int, int, int, int, int, void*);
 TQ_KERNEL(gated_part_norm, cf32, cptr, int, long long, cf32, float, void*, int, int, int, void*);
 TQ_KERNEL(add_rows, float*, cf32, long long, void*);
 TQ_QUERY(int, attention_masked_max_dim);

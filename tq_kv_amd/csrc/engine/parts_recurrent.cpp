@@ -59,6 +59,12 @@ std::string name_of(const Json& names, const char* role, const char* fallback) {
 TensorSpec matrix(int64_t a, int64_t b) { TensorSpec t; t.shape = {a, b}; return t; }
 TensorSpec vector_of(int64_t a, double std_dev = 0.02) { TensorSpec t; t.shape = {a}; t.std_dev = std_dev; return t; }
 
+// Steps that bring so many tokens of some sequence run their recurrences in chunks (three launches, every chunk a piece of work of its
+// own); shorter ones, steps of one token a sequence and the 32-bit path run them token by token, where the order of the sums does not
+// depend on how a sequence was cut.
+const int CHUNKED_FROM = 128;
+bool in_chunks(const StepContext& c, int dtype) { return dtype == BF16 && !c.all_decode && !c.capturing && c.max_new >= CHUNKED_FROM && !null_device(); }
+
 const void* at(const Tensor& t, int64_t column) { return (const char*)t.data + (size_t)column * dtype_size(t.dtype); }
 
 // ---- rglru -------------------------------------------------------------------------------------------
@@ -158,8 +164,18 @@ public:
         K::rglru_gates((const float*)u.data, (const float*)gate_a_->t.data, (const float*)gate_i_->t.data, (const float*)gate_a_b_->t.data,
                        (const float*)gate_i_b_->t.data, (const float*)decay_c_->t.data, (float*)a.data, (float*)g.data, (int)n, (int)width_, blocks_, c.stream);
         Tensor out = c.alloc(dtype, {n, width_});
-        K::linear_scan((const float*)a.data, (const float*)g.data, yx.data, dtype, 2 * width_, (const float*)y_bias_->t.data, state + conv_part, row,
-                       c.dev.cu, c.dev.seq_new, c.dev.seq_slot, out.data, c.n_seqs, (int)width_, c.stream);
+        if (in_chunks(c, dtype)) {
+            const Chunks ch = c.chunks(SCAN_CHUNK);
+            Tensor cp = c.alloc(F32, {ch.n, width_}), cl = c.alloc(F32, {ch.n, width_});
+            K::linear_chunks((const float*)a.data, (const float*)g.data, nullptr, dtype, 0, nullptr, ch.row0, ch.count, ch.n, (float*)cp.data, (float*)cl.data,
+                             nullptr, 1, (int)width_, c.stream);
+            K::chunk_carry((const float*)cp.data, width_, 1, (float*)cl.data, ch.seq_first, c.dev.seq_slot, state + conv_part, row, c.n_seqs, width_, c.stream);
+            K::linear_chunks((const float*)a.data, (const float*)g.data, yx.data, dtype, 2 * width_, (const float*)y_bias_->t.data, ch.row0, ch.count, ch.n,
+                             (float*)cp.data, (float*)cl.data, out.data, 2, (int)width_, c.stream);
+        } else {
+            K::linear_scan((const float*)a.data, (const float*)g.data, yx.data, dtype, 2 * width_, (const float*)y_bias_->t.data, state + conv_part, row,
+                           c.dev.cu, c.dev.seq_new, c.dev.seq_slot, out.data, c.n_seqs, (int)width_, c.stream);
+        }
         if (stream) {
             add_product(c, *stream, out, w_o_);
             return Tensor();
@@ -168,6 +184,7 @@ public:
     }
 
 private:
+    static const int SCAN_CHUNK = 32;
     int64_t hidden_, width_;
     int blocks_, taps_;
     double decay_scale_;
@@ -259,9 +276,24 @@ public:
                       c.dev.tok_seq, c.dev.tok_pos, c.dev.seq_slot, c.dev.seq_start, (float*)xbc.data, (int)n, (int)conv_ch_, c.stream);
         K::conv_state_update(at(zxbcdt, inner_), dtype, row_, nullptr, taps_, state, row, c.dev.cu, c.dev.seq_new, c.dev.seq_slot, c.n_seqs, (int)conv_ch_,
                              c.stream);
-        K::ssm_scan((const float*)xbc.data, conv_ch_, at(zxbcdt, inner_ + conv_ch_), dtype, row_, (const float*)dt_bias_->t.data, (const float*)a_log_->t.data,
-                    (const float*)d_->t.data, state + conv_part, row, c.dev.cu, c.dev.seq_new, c.dev.seq_slot, (float*)y.data, c.n_seqs, heads_, groups_,
-                    n_state_, p_dim_, c.stream);
+        if (in_chunks(c, dtype)) {
+            const Chunks ch = c.chunks(SCAN_CHUNK);
+            const int64_t per_head = (int64_t)n_state_ * p_dim_;
+            Tensor dt = c.alloc(F32, {n, heads_}), decay = c.alloc(F32, {n, heads_});
+            Tensor cs = c.alloc(F32, {ch.n, heads_, per_head}), cd = c.alloc(F32, {ch.n, heads_});
+            K::ssm_steps(at(zxbcdt, inner_ + conv_ch_), dtype, row_, (const float*)dt_bias_->t.data, (const float*)a_log_->t.data, (float*)dt.data,
+                         (float*)decay.data, (int)n, heads_, c.stream);
+            K::ssm_chunks((const float*)xbc.data, conv_ch_, (const float*)dt.data, (const float*)decay.data, (const float*)d_->t.data, ch.row0, ch.count, ch.n,
+                          (float*)cs.data, (float*)cd.data, nullptr, 1, heads_, groups_, n_state_, p_dim_, c.stream);
+            K::chunk_carry((const float*)cd.data, heads_, (int)per_head, (float*)cs.data, ch.seq_first, c.dev.seq_slot, state + conv_part, row, c.n_seqs,
+                           heads_ * per_head, c.stream);
+            K::ssm_chunks((const float*)xbc.data, conv_ch_, (const float*)dt.data, (const float*)decay.data, (const float*)d_->t.data, ch.row0, ch.count, ch.n,
+                          (float*)cs.data, (float*)cd.data, (float*)y.data, 2, heads_, groups_, n_state_, p_dim_, c.stream);
+        } else {
+            K::ssm_scan((const float*)xbc.data, conv_ch_, at(zxbcdt, inner_ + conv_ch_), dtype, row_, (const float*)dt_bias_->t.data, (const float*)a_log_->t.data,
+                        (const float*)d_->t.data, state + conv_part, row, c.dev.cu, c.dev.seq_new, c.dev.seq_slot, (float*)y.data, c.n_seqs, heads_, groups_,
+                        n_state_, p_dim_, c.stream);
+        }
         Tensor out = c.alloc(dtype, {n, inner_});
         K::gated_part_norm((const float*)y.data, zxbcdt.data, dtype, row_, (const float*)norm_w_->t.data, eps_, out.data, (int)n, (int)inner_, norm_groups_,
                            c.stream);
@@ -273,6 +305,7 @@ public:
     }
 
 private:
+    static const int SCAN_CHUNK = 64;
     int64_t hidden_, inner_, conv_ch_, total_, row_ = 0;
     int heads_, p_dim_, n_state_, groups_, taps_, norm_groups_;
     float eps_;

@@ -51,6 +51,7 @@ void StepContext::plan(const tqe_cache* cache, int n, const int32_t* slots, cons
         tables[(size_t)g].width = meta_[TQE_META_OFFSETS + 12 + TQE_MAX_GROUPS + g];
     }
     tiles_.clear();
+    chunks_.clear();
     memo.clear();
     carried.clear();
 }
@@ -111,6 +112,33 @@ Tiles StepContext::query_tiles(int tile) {
             reach.push_back((long long)host.tok_pos[host.cu[i] + a] + c);
         }
     return tiles_[key] = upload_tiles(seq, tok0, count, reach);
+}
+
+Chunks StepContext::chunks(int size) {
+    auto it = chunks_.find(size);
+    if (it != chunks_.end()) return it->second;
+    if (size < 1) raise(TQE_ERR_ARGUMENT, "chunks of %d tokens", size);
+    if (capturing) raise(TQE_ERR_STATE, "a part asked for chunks of the step while it was being captured as a graph (it is not graph_safe)");
+    std::vector<int32_t> row0, count, first;
+    for (int i = 0; i < n_seqs; ++i) {
+        first.push_back((int32_t)row0.size());
+        for (int a = 0; a < lens[(size_t)i]; a += size) {
+            row0.push_back(host.cu[i] + a);
+            count.push_back(std::min(size, lens[(size_t)i] - a));
+        }
+    }
+    first.push_back((int32_t)row0.size());
+    Chunks c;
+    c.n = (int)row0.size();
+    std::vector<int32_t> all(row0);
+    all.insert(all.end(), count.begin(), count.end());
+    all.insert(all.end(), first.begin(), first.end());
+    int32_t* dev_mem = (int32_t*)ws->alloc_for_step(all.size() * sizeof(int32_t));       // later layers read them too
+    staging->upload(dev_mem, all.data(), all.size() * sizeof(int32_t), stream);
+    c.row0 = dev_mem;
+    c.count = dev_mem + c.n;
+    c.seq_first = dev_mem + 2 * (size_t)c.n;
+    return chunks_[size] = c;
 }
 
 Tiles StepContext::last_tiles(int tile) {

@@ -38,6 +38,15 @@ struct Tiles {
     int n = 0;
 };
 
+// The step's tokens cut into chunks of up to `size` consecutive tokens of one sequence, sequence by sequence and in order: chunk c is
+// packed rows row0[c] .. + count[c]; sequence s owns chunks seq_first[s] .. seq_first[s + 1] (all on the device).
+struct Chunks {
+    const int32_t* row0 = nullptr;
+    const int32_t* count = nullptr;
+    const int32_t* seq_first = nullptr;
+    int n = 0;
+};
+
 struct StepShape {
     int n_tokens, n_seqs, n_want;
     std::vector<int> widths;
@@ -84,6 +93,9 @@ struct StepContext {
     Tiles query_tiles(int tile);
     // The same for the step's last_rows, in their own numbering.
     Tiles last_tiles(int tile);
+    // The step's tokens in chunks of a sequence's consecutive tokens, for mixers that run a recurrence piece by piece; built and
+    // uploaded when a mixer first asks for this size (not while a step is captured).
+    Chunks chunks(int size);
 
     Tensor alloc(int dtype, std::initializer_list<int64_t> dims) { return ws->tensor(dtype, dims); }
 
@@ -96,6 +108,7 @@ struct StepContext {
     ~StepContext();
 private:
     std::map<std::pair<int, int>, Tiles> tiles_;
+    std::map<int, Chunks> chunks_;
     Tiles upload_tiles(std::vector<int32_t>& seq, std::vector<int32_t>& tok0, std::vector<int32_t>& count, const std::vector<long long>& reach);
     void carve(StepArrays& out, const int32_t* base, const int32_t* meta);
     int32_t meta_[TQE_META_SIZE];

@@ -203,6 +203,174 @@ void ssm_scan_kernel(const float* __restrict__ xbc, long long xbc_stride, const 
     }
 }
 
+// ---- long steps: the recurrences in chunks ---------------------------------------------------------------------------
+// A step that brings many tokens of a sequence is cut into chunks of consecutive tokens of one sequence (chunk c: packed rows
+// chunk_row0[c] .. + chunk_count[c]; the chunks of sequence s are seq_first[s] .. seq_first[s + 1], in order).  Three launches:
+// every chunk runs its recurrence from a zero state and leaves its last state and the product of its decays; a carry pass walks a
+// sequence's chunks in order, S <- decay S + local, and leaves in each chunk's place the state the chunk starts from (the
+// sequence's state row gets the last one); every chunk runs again from that state and writes the outputs.  Twice the arithmetic,
+// but as many independent pieces of work as there are chunks, where the plain kernels above have one per sequence.
+enum { CHUNK_LOCAL = 1, CHUNK_APPLY = 2 };
+
+template <typename TA, int MODE>
+__global__ __launch_bounds__(256)
+void linear_chunk_kernel(const float* __restrict__ a, const float* __restrict__ g, const TA* __restrict__ y, long long y_stride,
+                         const float* __restrict__ y_bias, const int32_t* __restrict__ chunk_row0, const int32_t* __restrict__ chunk_count,
+                         float* __restrict__ chunk_p, float* __restrict__ chunk_l, TA* __restrict__ out, int width) {
+    const int c = blockIdx.y;
+    const int ch = blockIdx.x * blockDim.x + threadIdx.x;
+    if (ch >= width) return;
+    const int t0 = chunk_row0[c], n = chunk_count[c];
+    float S = MODE == CHUNK_APPLY ? chunk_l[(size_t)c * width + ch] : 0.f, P = 1.f;
+    const float yb = (MODE == CHUNK_APPLY && y_bias) ? y_bias[ch] : 0.f;
+    for (int j = 0; j < n; ++j) {
+        const size_t at = (size_t)(t0 + j) * width + ch;
+        const float av = a[at];
+        S = fmaf(av, S, g[at]);
+        if (MODE == CHUNK_LOCAL) P *= av;
+        else out[at] = from_float<TA>(S * gelu_tanh_f(to_float(y[(size_t)(t0 + j) * y_stride + ch]) + yb));
+    }
+    if (MODE == CHUNK_LOCAL) {
+        chunk_p[(size_t)c * width + ch] = P;
+        chunk_l[(size_t)c * width + ch] = S;
+    }
+}
+
+// elements: per sequence `per_seq` state values; element e of a chunk decays with chunk_p[c * p_stride + e / p_div]
+__global__ __launch_bounds__(256)
+void chunk_carry_kernel(const float* __restrict__ chunk_p, long long p_stride, int p_div, float* __restrict__ chunk_l, const int32_t* __restrict__ seq_first,
+                        const int32_t* __restrict__ seq_slot, float* __restrict__ state, long long state_stride, long long per_seq) {
+    const int s = blockIdx.y;
+    const long long e = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+    if (e >= per_seq) return;
+    const int c0 = seq_first[s], c1 = seq_first[s + 1];
+    if (c1 <= c0) return;
+    float* st = state + (size_t)seq_slot[s] * state_stride + e;
+    float S = *st;
+    for (int c = c0; c < c1; ++c) {
+        float* l = chunk_l + (size_t)c * per_seq + e;
+        const float local = *l;
+        *l = S;
+        S = fmaf(chunk_p[(size_t)c * p_stride + e / p_div], S, local);
+    }
+    *st = S;
+}
+
+// dt = softplus(raw + bias) and the decay exp(-exp(a_log) dt) of every (token, head), once
+template <typename TA>
+__global__ __launch_bounds__(256)
+void ssm_steps_kernel(const TA* __restrict__ dt_raw, long long dt_stride, const float* __restrict__ dt_bias, const float* __restrict__ a_log,
+                      float* __restrict__ dt_out, float* __restrict__ decay_out, long long n, int heads) {
+    const long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= n) return;
+    const long long t = i / heads;
+    const int h = (int)(i % heads);
+    const float dt = softplus_f(to_float(dt_raw[t * dt_stride + h]) + dt_bias[h]);
+    dt_out[i] = dt;
+    decay_out[i] = expf(-expf(a_log[h]) * dt);
+}
+
+__device__ __forceinline__ float dpp_quad_xor1(float v) { return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0xB1, 0xf, 0xf, false)); }
+__device__ __forceinline__ float dpp_quad_xor2(float v) { return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x4E, 0xf, 0xf, false)); }
+__device__ __forceinline__ float dpp_half_mirror(float v) { return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x141, 0xf, 0xf, false)); }
+__device__ __forceinline__ float dpp_row_mirror(float v) { return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x140, 0xf, 0xf, false)); }
+// the sum over a row of 16 lanes, in every lane of the row, in one fixed order
+__device__ __forceinline__ float row16_sum(float v) {
+    v += dpp_quad_xor1(v);
+    v += dpp_quad_xor2(v);
+    v += dpp_half_mirror(v);
+    v += dpp_row_mirror(v);
+    return v;
+}
+
+// A block of four waves per (chunk, head, 64 columns of the head's values); a wave takes 16 columns.  Lane = 16 * column group +
+// row group: a lane keeps RN consecutive rows of 4 consecutive columns of the state, so a token costs it RN values each of B and
+// C and 4 of x for 4 RN products; a column's output is summed over the 16 row groups, which are one row of lanes.
+// vec: rows and columns fall into pieces of four floats at aligned places (the host says so).
+template <int RN, int MODE>
+__global__ __launch_bounds__(256)
+void ssm_chunk_kernel(const float* __restrict__ xbc, long long xbc_stride, const float* __restrict__ dt, const float* __restrict__ decay,
+                      const float* __restrict__ d_skip, const int32_t* __restrict__ chunk_row0, const int32_t* __restrict__ chunk_count,
+                      float* __restrict__ chunk_state, float* __restrict__ chunk_decay, float* __restrict__ y_out, int heads, int groups,
+                      int n_state, int p_dim, int vec) {
+    const int c = blockIdx.z, h = blockIdx.y;
+    const int wave = threadIdx.x / TQK_WAVE, lane = threadIdx.x % TQK_WAVE;
+    const int rowgroup = lane & 15, colgroup = lane >> 4;
+    const int p0 = (blockIdx.x * 4 + wave) * 16 + colgroup * 4, r0 = rowgroup * RN;
+    if ((blockIdx.x * 4 + wave) * 16 >= p_dim) return;
+    const int t0 = chunk_row0[c], n = chunk_count[c];
+    const int inner = heads * p_dim, grp = h / (heads / groups);
+    float* cs = chunk_state + ((size_t)c * heads + h) * n_state * p_dim;
+    float S[RN][4];
+#pragma unroll
+    for (int i = 0; i < RN; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+            S[i][j] = (MODE == CHUNK_APPLY && r0 + i < n_state && p0 + j < p_dim) ? cs[(size_t)(r0 + i) * p_dim + p0 + j] : 0.f;
+    const float dsk = d_skip[h];
+    float total = 1.f;
+    for (int k = 0; k < n; ++k) {
+        const size_t t = (size_t)(t0 + k);
+        const float* row = xbc + t * xbc_stride;
+        const float dtv = dt[t * heads + h], dec = decay[t * heads + h];
+        const float* xs = row + (size_t)h * p_dim + p0;
+        const float* Bs = row + inner + (size_t)grp * n_state + r0;
+        const float* Cs = Bs + (size_t)groups * n_state;
+        float x[4], B[RN], C[RN];
+        if (vec) {
+            const float4 xv = *reinterpret_cast<const float4*>(xs);
+            x[0] = xv.x; x[1] = xv.y; x[2] = xv.z; x[3] = xv.w;
+#pragma unroll
+            for (int i = 0; i < RN; i += 4) {
+                const float4 b = *reinterpret_cast<const float4*>(Bs + i);
+                B[i] = b.x; B[i + 1 < RN ? i + 1 : i] = b.y; B[i + 2 < RN ? i + 2 : i] = b.z; B[i + 3 < RN ? i + 3 : i] = b.w;
+                if (MODE == CHUNK_APPLY) {
+                    const float4 cv = *reinterpret_cast<const float4*>(Cs + i);
+                    C[i] = cv.x; C[i + 1 < RN ? i + 1 : i] = cv.y; C[i + 2 < RN ? i + 2 : i] = cv.z; C[i + 3 < RN ? i + 3 : i] = cv.w;
+                }
+            }
+        } else {
+#pragma unroll
+            for (int j = 0; j < 4; ++j) x[j] = p0 + j < p_dim ? xs[j] : 0.f;
+#pragma unroll
+            for (int i = 0; i < RN; ++i) {
+                B[i] = r0 + i < n_state ? Bs[i] : 0.f;
+                if (MODE == CHUNK_APPLY) C[i] = r0 + i < n_state ? Cs[i] : 0.f;
+            }
+        }
+        float dx[4], acc[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int j = 0; j < 4; ++j) dx[j] = dtv * x[j];
+#pragma unroll
+        for (int i = 0; i < RN; ++i)
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                S[i][j] = fmaf(dec, S[i][j], B[i] * dx[j]);
+                if (MODE == CHUNK_APPLY) acc[j] = fmaf(S[i][j], C[i], acc[j]);
+            }
+        if (MODE == CHUNK_APPLY) {
+#pragma unroll
+            for (int j = 0; j < 4; ++j) acc[j] = fmaf(dsk, x[j], row16_sum(acc[j]));
+            if (rowgroup == 0) {
+                float* yo = y_out + t * inner + (size_t)h * p_dim + p0;
+                if (vec) *reinterpret_cast<float4*>(yo) = make_float4(acc[0], acc[1], acc[2], acc[3]);
+                else
+#pragma unroll
+                    for (int j = 0; j < 4; ++j)
+                        if (p0 + j < p_dim) yo[j] = acc[j];
+            }
+        } else total *= dec;
+    }
+    if (MODE == CHUNK_LOCAL) {
+#pragma unroll
+        for (int i = 0; i < RN; ++i)
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+                if (r0 + i < n_state && p0 + j < p_dim) cs[(size_t)(r0 + i) * p_dim + p0 + j] = S[i][j];
+        if (blockIdx.x == 0 && threadIdx.x == 0) chunk_decay[(size_t)c * heads + h] = total;
+    }
+}
+
 // ---- gate, then norm in parts --------------------------------------------------------------------------------
 // v = y silu(z); every one of `parts` equal parts of a row is divided by its own root mean square; times w.  A block per
 // (token, part).
@@ -329,6 +497,76 @@ extern "C" int tqk_ssm_scan(const float* xbc, long long xbc_stride, const void* 
 #undef TQK_SSM_BY_SIZE
 #undef TQK_SSM
     return tqk_check_launch("tqk_ssm_scan");
+}
+
+extern "C" int tqk_linear_chunks(const float* a, const float* g, const void* y, int act_dtype, long long y_stride, const float* y_bias,
+                                 const int32_t* chunk_row0, const int32_t* chunk_count, int n_chunks, float* chunk_p, float* chunk_l, void* out, int mode,
+                                 int width, void* stream) {
+    TQK_REQUIRE(a && g && chunk_row0 && chunk_count && chunk_p && chunk_l, "tqk_linear_chunks: null pointer");
+    TQK_REQUIRE(mode == CHUNK_LOCAL || (mode == CHUNK_APPLY && y && out && y_stride >= width), "tqk_linear_chunks: mode %d, or nothing to write to", mode);
+    TQK_REQUIRE(n_chunks >= 0 && n_chunks <= 65535 && width > 0, "tqk_linear_chunks: bad sizes");
+    if (n_chunks == 0) return 0;
+    hipStream_t s = (hipStream_t)stream;
+    dim3 grid((width + 255) / 256, n_chunks);
+#define TQK_LC(TA, MODE) linear_chunk_kernel<TA, MODE><<<grid, 256, 0, s>>>(a, g, (const TA*)y, y_stride, y_bias, chunk_row0, chunk_count, chunk_p, chunk_l, (TA*)out, width)
+    if (mode == CHUNK_LOCAL) TQK_LC(float, CHUNK_LOCAL);
+    else if (act_dtype == TQK_F32) TQK_LC(float, CHUNK_APPLY);
+    else if (act_dtype == TQK_BF16) TQK_LC(bf16_t, CHUNK_APPLY);
+    else return tqk_fail("tqk_linear_chunks: unknown dtype %d", act_dtype);
+#undef TQK_LC
+    return tqk_check_launch("tqk_linear_chunks");
+}
+
+extern "C" int tqk_chunk_carry(const float* chunk_p, long long p_stride, int p_div, float* chunk_l, const int32_t* seq_first, const int32_t* seq_slot,
+                               float* state, long long state_stride, int n_seqs, long long per_seq, void* stream) {
+    TQK_REQUIRE(chunk_p && chunk_l && seq_first && seq_slot && state, "tqk_chunk_carry: null pointer");
+    TQK_REQUIRE(n_seqs >= 0 && n_seqs <= 65535 && per_seq > 0 && p_div > 0 && state_stride >= per_seq, "tqk_chunk_carry: bad sizes");
+    if (n_seqs == 0) return 0;
+    const long long blocks = (per_seq + 255) / 256;
+    TQK_REQUIRE(blocks <= 0x7fffffff, "tqk_chunk_carry: too many elements");
+    dim3 grid((unsigned)blocks, n_seqs);
+    chunk_carry_kernel<<<grid, 256, 0, (hipStream_t)stream>>>(chunk_p, p_stride, p_div, chunk_l, seq_first, seq_slot, state, state_stride, per_seq);
+    return tqk_check_launch("tqk_chunk_carry");
+}
+
+extern "C" int tqk_ssm_steps(const void* dt_raw, int dt_dtype, long long dt_stride, const float* dt_bias, const float* a_log, float* dt_out,
+                             float* decay_out, int n_tokens, int heads, void* stream) {
+    TQK_REQUIRE(dt_raw && dt_bias && a_log && dt_out && decay_out, "tqk_ssm_steps: null pointer");
+    TQK_REQUIRE(n_tokens >= 0 && heads > 0 && dt_stride >= heads, "tqk_ssm_steps: bad sizes");
+    const long long n = (long long)n_tokens * heads;
+    if (n == 0) return 0;
+    const long long blocks = (n + 255) / 256;
+    TQK_REQUIRE(blocks <= 0x7fffffff, "tqk_ssm_steps: too many elements");
+    hipStream_t s = (hipStream_t)stream;
+    if (dt_dtype == TQK_F32) ssm_steps_kernel<float><<<(unsigned)blocks, 256, 0, s>>>((const float*)dt_raw, dt_stride, dt_bias, a_log, dt_out, decay_out, n, heads);
+    else if (dt_dtype == TQK_BF16) ssm_steps_kernel<bf16_t><<<(unsigned)blocks, 256, 0, s>>>((const bf16_t*)dt_raw, dt_stride, dt_bias, a_log, dt_out, decay_out, n, heads);
+    else return tqk_fail("tqk_ssm_steps: unknown dtype %d", dt_dtype);
+    return tqk_check_launch("tqk_ssm_steps");
+}
+
+extern "C" int tqk_ssm_chunks(const float* xbc, long long xbc_stride, const float* dt, const float* decay, const float* d_skip, const int32_t* chunk_row0,
+                              const int32_t* chunk_count, int n_chunks, float* chunk_state, float* chunk_decay, float* y_out, int mode, int heads,
+                              int groups, int n_state, int p_dim, void* stream) {
+    TQK_REQUIRE(xbc && dt && decay && d_skip && chunk_row0 && chunk_count && chunk_state && chunk_decay, "tqk_ssm_chunks: null pointer");
+    TQK_REQUIRE(mode == CHUNK_LOCAL || (mode == CHUNK_APPLY && y_out), "tqk_ssm_chunks: mode %d, or nothing to write to", mode);
+    TQK_REQUIRE(n_chunks >= 0 && n_chunks <= 65535 && heads > 0 && heads <= 65535 && groups > 0 && heads % groups == 0 && n_state > 0 && p_dim > 0,
+                "tqk_ssm_chunks: bad sizes (%d heads in %d groups)", heads, groups);
+    TQK_REQUIRE(n_state <= 256, "tqk_ssm_chunks: a state of %d rows, the kernel takes up to 256", n_state);
+    TQK_REQUIRE(xbc_stride >= (long long)heads * p_dim + 2LL * groups * n_state, "tqk_ssm_chunks: stride too short");
+    if (n_chunks == 0) return 0;
+    hipStream_t s = (hipStream_t)stream;
+    const int rn = n_state <= 16 ? 1 : n_state <= 32 ? 2 : n_state <= 64 ? 4 : n_state <= 128 ? 8 : 16;
+    // pieces of four floats at aligned places: whole rows of four per lane, columns and the row's parts at multiples of four
+    const int vec = (rn % 4 == 0 && n_state == 16 * rn && p_dim % 16 == 0 && xbc_stride % 4 == 0 && ((uintptr_t)xbc & 15) == 0 && ((uintptr_t)y_out & 15) == 0) ? 1 : 0;
+    dim3 grid((p_dim + 63) / 64, heads, n_chunks);
+#define TQK_SC(RN, MODE) ssm_chunk_kernel<RN, MODE><<<grid, 256, 0, s>>>(xbc, xbc_stride, dt, decay, d_skip, chunk_row0, chunk_count, chunk_state, chunk_decay, \
+        y_out, heads, groups, n_state, p_dim, vec)
+#define TQK_SC_BY_SIZE(MODE) do { if (rn == 1) TQK_SC(1, MODE); else if (rn == 2) TQK_SC(2, MODE); else if (rn == 4) TQK_SC(4, MODE); \
+        else if (rn == 8) TQK_SC(8, MODE); else TQK_SC(16, MODE); } while (0)
+    if (mode == CHUNK_LOCAL) TQK_SC_BY_SIZE(CHUNK_LOCAL); else TQK_SC_BY_SIZE(CHUNK_APPLY);
+#undef TQK_SC_BY_SIZE
+#undef TQK_SC
+    return tqk_check_launch("tqk_ssm_chunks");
 }
 
 extern "C" int tqk_gated_part_norm(const float* y, const void* z, int act_dtype, long long z_stride, const float* w, float eps, void* out, int n_tokens,

@@ -350,6 +350,22 @@ int tqk_ssm_max_state(void);
 int tqk_ssm_scan(const float* xbc, long long xbc_stride, const void* dt_raw, int dt_dtype, long long dt_stride, const float* dt_bias,
                  const float* a_log, const float* d_skip, float* state, long long state_stride, const int32_t* cu, const int32_t* seq_new,
                  const int32_t* seq_slot, float* y_out, int n_seqs, int heads, int groups, int n_state, int p_dim, void* stream);
+/* The same recurrences for steps that bring many tokens of a sequence, in chunks of consecutive tokens of one sequence (chunk c: packed rows
+ * chunk_row0[c] .. + chunk_count[c]; sequence s owns chunks seq_first[s] .. seq_first[s + 1], in order).  mode 1: every chunk from a zero
+ * state; its last state goes to chunk_l / chunk_state, the product of its decays to chunk_p / chunk_decay.  tqk_chunk_carry: per sequence
+ * S <- p S + local over its chunks, from the sequence's state row, leaving in each chunk's place the state it starts from and in the state
+ * row the last (element e of per_seq decays with chunk_p[c * p_stride + e / p_div]).  mode 2: every chunk again from that state, writing
+ * the outputs.  tqk_ssm_steps: dt = softplus(raw + bias) and decay = exp(-exp(a_log) dt) per (token, head), which tqk_ssm_chunks takes. */
+int tqk_linear_chunks(const float* a, const float* g, const void* y, int act_dtype, long long y_stride, const float* y_bias,
+                      const int32_t* chunk_row0, const int32_t* chunk_count, int n_chunks, float* chunk_p, float* chunk_l, void* out, int mode,
+                      int width, void* stream);
+int tqk_chunk_carry(const float* chunk_p, long long p_stride, int p_div, float* chunk_l, const int32_t* seq_first, const int32_t* seq_slot,
+                    float* state, long long state_stride, int n_seqs, long long per_seq, void* stream);
+int tqk_ssm_steps(const void* dt_raw, int dt_dtype, long long dt_stride, const float* dt_bias, const float* a_log, float* dt_out,
+                  float* decay_out, int n_tokens, int heads, void* stream);
+int tqk_ssm_chunks(const float* xbc, long long xbc_stride, const float* dt, const float* decay, const float* d_skip, const int32_t* chunk_row0,
+                   const int32_t* chunk_count, int n_chunks, float* chunk_state, float* chunk_decay, float* y_out, int mode, int heads,
+                   int groups, int n_state, int p_dim, void* stream);
 /* out = norm_parts(y silu(z)) w: `parts` equal parts of a row, each divided by its own root mean square. */
 int tqk_gated_part_norm(const float* y, const void* z, int act_dtype, long long z_stride, const float* w, float eps, void* out, int n_tokens,
                         int size, int parts, void* stream);
