@@ -28,6 +28,7 @@ TQ_KERNEL(fused_store, cptr, ci32, cf32, int, float, cptr, int, void*, int, int,
 TQ_KERNEL(fused_gated, cptr, cf32, int, float, cptr, int, void*, int, int, int, void*);
 TQ_QUERY(int, fused_residual_parts, int, int);
 TQ_KERNEL(fused_residual, cptr, cptr, int, float*, cptr, void*, float*, int, int, int, void*);
+TQ_KERNEL(fused_residual_wf32, cptr, cptr, int, float*, cf32, void*, float*, int, int, int, void*);
 TQ_KERNEL(fused_qkv, cptr, cf32, int, float, cptr, int, cptr, cf32, cf32, int, ci32, ci32, int, void*, void*, int, void*, int, int, int, int,
           int, void*);
 TQ_QUERY(int, mid_splits, int, int, int);

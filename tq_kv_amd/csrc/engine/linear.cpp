@@ -298,8 +298,12 @@ void add_product(StepContext& c, Stream& stream, const Tensor& x, const Weight& 
     if (stream.ss_buffer.defined() && stream.ss_buffer.numel() < (int64_t)parts * 16)
         raise(TQE_ERR_STATE, "the stream's buffer for sums of squares holds %lld values, %d pieces of 16 are written",
               (long long)stream.ss_buffer.numel(), parts);
-    K::fused_residual(x.data, wp, packed, (float*)stream.h.data, norm ? norm->fold_weight()->data : nullptr, stream.xw_buffer.data,
-                      (float*)stream.ss_buffer.data, (int)x.shape[0], (int)w.n, (int)w.k, c.stream);
+    if (norm && norm->fold_weight()->dtype == F32)
+        K::fused_residual_wf32(x.data, wp, packed, (float*)stream.h.data, (const float*)norm->fold_weight()->data, stream.xw_buffer.data,
+                               (float*)stream.ss_buffer.data, (int)x.shape[0], (int)w.n, (int)w.k, c.stream);
+    else
+        K::fused_residual(x.data, wp, packed, (float*)stream.h.data, norm ? norm->fold_weight()->data : nullptr, stream.xw_buffer.data,
+                          (float*)stream.ss_buffer.data, (int)x.shape[0], (int)w.n, (int)w.k, c.stream);
     stream.n_ss = parts;
     stream.xw_for = norm;
     stream.pending = Pending();

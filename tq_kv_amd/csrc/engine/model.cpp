@@ -143,7 +143,8 @@ Tensor Model::forward(StepContext& c, const CacheStore& cache, float* out) {
     if (c.fuse_small) {
         stream.xw_buffer = c.alloc(BF16, {c.n_tokens, s.hidden_size});
         stream.ss_buffer = c.alloc(F32, {(s.hidden_size + 15) / 16, 16});        // the most pieces a product gives
-        const Norm* norm = firsts[0] && firsts[0]->foldable() ? firsts[0] : nullptr;
+        // (the gather multiplies by a bfloat16 weight; a first norm whose weight is kept in 32 bits runs as a kernel of its own)
+        const Norm* norm = firsts[0] && firsts[0]->foldable() && firsts[0]->fold_weight()->dtype == BF16 ? firsts[0] : nullptr;
         K::embed(table.data, table.dtype, c.dev.tokens, c.n_tokens, (int)s.hidden_size, (int)s.vocab_size, scale, (float*)h.data,
                  stream.xw_buffer.data, norm ? norm->fold_weight()->data : nullptr, (float*)stream.ss_buffer.data, c.stream);
         stream.xw_for = norm;

@@ -145,7 +145,8 @@ public:
         k_add_rmsnorm(c, (float*)h.data, delta, weight_->t, eps_, rows, n_rows, h.shape[0], out, false);
     }
     bool takes_partial_sums() const override { return true; }
-    bool foldable() const override { return weight_ && weight_->t.dtype == BF16; }
+    // (the weight as stored, bfloat16, or the sum 1 + w, float32: the kernels that prepare a norm take either)
+    bool foldable() const override { return weight_ && (weight_->t.dtype == BF16 || (unit_offset_ && weight_->t.dtype == F32)); }
     const Tensor* fold_weight() const override { return &weight_->t; }
     float fold_eps() const override { return eps_; }
 

@@ -195,6 +195,9 @@ void skinny_fused_kernel(const FusedArgs p) {
     const int ml = m < p.M ? m : 0;
     float4 pre_f0[TILES], pre_f1 = make_float4(0.f, 0.f, 0.f, 0.f);
     uint2 pre_h0[TILES], pre_h1 = make_uint2(0, 0);
+    // (EPI_RESIDUAL with TY = float: the next norm's weight is float32, four values a tile)
+    constexpr bool WIDE_NORM_W = EPI == EPI_RESIDUAL && sizeof(TY) == 4;
+    float4 pre_wf[WIDE_NORM_W ? TILES : 1];
 #pragma unroll
     for (int t = 0; t < TILES; ++t) { pre_f0[t] = pre_f1; pre_h0[t] = pre_h1; }
     int pos = 0, page = -1;
@@ -215,7 +218,8 @@ void skinny_fused_kernel(const FusedArgs p) {
             for (int t = 0; t < TILES; ++t) {
                 const int n = min(n_lo0 + 16 * t + nb, p.N - 4);
                 pre_f0[t] = *reinterpret_cast<const float4*>(p.h + (size_t)ml * p.N + n);
-                pre_h0[t] = *reinterpret_cast<const uint2*>(p.next_norm_w ? p.next_norm_w + n : p.w);
+                if constexpr (WIDE_NORM_W) pre_wf[t] = *reinterpret_cast<const float4*>(p.next_norm_w ? reinterpret_cast<const float*>(p.next_norm_w) + n : p.h);
+                else pre_h0[t] = *reinterpret_cast<const uint2*>(p.next_norm_w ? p.next_norm_w + n : p.w);
             }
         }
         if (EPI == EPI_QKV) {
@@ -329,8 +333,9 @@ void skinny_fused_kernel(const FusedArgs p) {
 #pragma unroll
             for (int t = 0; t < TILES; ++t) {
                 const float pre_h[4] = {pre_f0[t].x, pre_f0[t].y, pre_f0[t].z, pre_f0[t].w};
-                const float pre_w[4] = {__uint_as_float(pre_h0[t].x << 16), __uint_as_float(pre_h0[t].x & 0xffff0000u),
-                                        __uint_as_float(pre_h0[t].y << 16), __uint_as_float(pre_h0[t].y & 0xffff0000u)};
+                float pre_w[4] = {__uint_as_float(pre_h0[t].x << 16), __uint_as_float(pre_h0[t].x & 0xffff0000u),
+                                  __uint_as_float(pre_h0[t].y << 16), __uint_as_float(pre_h0[t].y & 0xffff0000u)};
+                if constexpr (WIDE_NORM_W) { pre_w[0] = pre_wf[t].x; pre_w[1] = pre_wf[t].y; pre_w[2] = pre_wf[t].z; pre_w[3] = pre_wf[t].w; }
 #pragma unroll
                 for (int r = 0; r < 4; ++r) {
                     const int n = n_lo0 + 16 * t + nb + r;
@@ -509,6 +514,20 @@ extern "C" int tqk_fused_residual(const void* x, const void* w, int w_packed, fl
     TQK_REQUIRE(((((uintptr_t)h) | ((uintptr_t)next_norm_w)) & 15) == 0, "tqk_fused_residual: h and the norm's weight must be 16-byte aligned");
     if (M == 0) return 0;
     return launch_tiled<false, EPI_RESIDUAL, bf16_t>(a, (hipStream_t)stream);
+}
+
+/* The same with the next norm's weight in float32 (a norm that multiplies by 1 + w keeps that sum in 32 bits). */
+extern "C" int tqk_fused_residual_wf32(const void* x, const void* w, int w_packed, float* h, const float* next_norm_w, void* xw_out,
+                                       float* ss_out, int M, int N, int K, void* stream) {
+    FusedArgs a = {};
+    a.x = (const bf16_t*)x; a.w = (const bf16_t*)w; a.w_packed = w_packed; a.M = M; a.N = N; a.K = K; a.h = h;
+    a.next_norm_w = (const bf16_t*)(const void*)next_norm_w; a.xw_out = (bf16_t*)xw_out; a.ss_out = ss_out;
+    if (check_common(a, "tqk_fused_residual_wf32")) return -1;
+    TQK_REQUIRE(h && xw_out && next_norm_w, "tqk_fused_residual_wf32: null pointer");
+    TQK_REQUIRE(N % 4 == 0, "tqk_fused_residual_wf32: N=%d must be a multiple of 4", N);
+    TQK_REQUIRE(((((uintptr_t)h) | ((uintptr_t)next_norm_w)) & 15) == 0, "tqk_fused_residual_wf32: h and the norm's weight must be 16-byte aligned");
+    if (M == 0) return 0;
+    return launch_tiled<false, EPI_RESIDUAL, float>(a, (hipStream_t)stream);
 }
 
 /* The q, k, v product of a decoding step: the (normalised) product + bias, q and k rotated

@@ -95,6 +95,8 @@ int tqk_fused_gated(const void* x, const float* ss_parts, int n_ss_parts, float 
 /* h[M,N] += bfloat16(x w^T) in float32; xw_out = bfloat16(h * next_norm_w) or bfloat16(h);
  * ss_out (optional) [tqk_fused_residual_parts(N, K), 16] */
 int tqk_fused_residual_parts(int N, int K);
+int tqk_fused_residual_wf32(const void* x, const void* w, int w_packed, float* h, const float* next_norm_w, void* xw_out,
+                            float* ss_out, int M, int N, int K, void* stream);        /* the same, the norm's weight in float32 */
 int tqk_fused_residual(const void* x, const void* w, int w_packed, float* h, const void* next_norm_w, void* xw_out,
                        float* ss_out, int M, int N, int K, void* stream);
 /* q, k, v of a decoding step: + bias, rotation (halves over the whole head) at tok_pos[m],
