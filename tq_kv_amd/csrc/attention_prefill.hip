@@ -102,6 +102,7 @@ struct PrefillArgs {
     const int32_t* seq_new;
     int window;
     float scale;
+    float cap;               // > 0: scores become cap tanh(scale s / cap)
     bf16_t* out;
     int n_heads, n_kv_heads, n_tiles;
     int tq_shift;            // log2 of the queries per tile
@@ -123,6 +124,7 @@ struct Wave {
     int wave_first, wave_last, wave_lo, wave_lo_last;
     int seq_end, last_page;
     float c2;
+    float cap_in, cap_c2;                        // CAP: scale / cap, and cap log2 e
     const bf16_t* keys;
     const bf16_t* values;
     size_t page_stride;
@@ -173,7 +175,13 @@ __device__ __forceinline__ void stage_page(const Wave<D>& w, const u32x4_t (&kr)
 }
 
 // The work on one page, held in kc, vc.
-template <int D, int SPLIT>
+// tanh by one exponential: 1 - 2 / (e^(2x) + 1); exact at both ends (e^(2x) = inf gives 1, 0 gives -1)
+__device__ __forceinline__ float pf_tanh(float x) {
+    const float e = __builtin_amdgcn_exp2f(x * 2.88539008177792681472f);
+    return 1.f - 2.f * __builtin_amdgcn_rcpf(e + 1.f);
+}
+
+template <int D, int SPLIT, bool CAP>
 __device__ __forceinline__ void page_step(Wave<D>& w, int pg, int page_now, lds_byte* __restrict__ kc, lds_byte* __restrict__ vc) {
     using L = Layout<D>;
     constexpr int KS = Wave<D>::KS, DT = Wave<D>::DT;
@@ -218,6 +226,11 @@ __device__ __forceinline__ void page_step(Wave<D>& w, int pg, int page_now, lds_
         __builtin_amdgcn_sched_barrier(0);
         // the mask is needed only on tiles that cross a query's causal or window edge
         const bool need_mask = k0 + 31 > w.wave_first || k0 < w.wave_lo_last;
+        if (CAP) {
+            // the capped score, already in powers of two (the mask comes after: tanh of -inf is -1)
+#pragma unroll
+            for (int i = 0; i < 16; ++i) s[i] = w.cap_c2 * pf_tanh(s[i] * w.cap_in);
+        }
         if (need_mask) {
 #pragma unroll
             for (int i = 0; i < 16; ++i) {
@@ -231,7 +244,7 @@ __device__ __forceinline__ void page_step(Wave<D>& w, int pg, int page_now, lds_
         // is taken of these, not of the raw scores: a product of the matrix cores would have to be made canonical
         // value by value before a maximum may look at it.)
 #pragma unroll
-        for (int i = 0; i < 16; ++i) s[i] = fmaf(s[i], w.c2, -w.m);
+        for (int i = 0; i < 16; ++i) s[i] = CAP ? s[i] - w.m : fmaf(s[i], w.c2, -w.m);
         float mx = -INFINITY;
 #pragma unroll
         for (int i = 0; i < 16; i += 2) mx = fmaxf(mx, fmaxf(s[i], s[i + 1]));
@@ -286,7 +299,7 @@ __device__ __forceinline__ void page_step(Wave<D>& w, int pg, int page_now, lds_
 #define PF_SPLIT_COL_WAVES 4
 #define PF_HANDOVER_BYTES (18 * PF_SPLIT_COL_WAVES * TQK_WAVE * 4)
 
-template <int D, int SPLIT>
+template <int D, int SPLIT, bool CAP>
 __global__ __launch_bounds__(PF_MAX_WAVES * TQK_WAVE)
 void attention_prefill_kernel(const PrefillArgs p) {
     using L = Layout<D>;
@@ -349,6 +362,8 @@ void attention_prefill_kernel(const PrefillArgs p) {
     w.wave_lo = p.window > 0 ? max(0, w.wave_first - p.window + 1) : 0;            // first key any of its queries sees
     w.wave_lo_last = p.window > 0 ? max(0, w.wave_last - p.window + 1) : 0;        // first key all of them see
     w.c2 = p.scale * 1.44269504088896340736f;
+    w.cap_in = CAP ? p.scale / p.cap : 0.f;
+    w.cap_c2 = p.cap * 1.44269504088896340736f;
     const int tile_lo = p.window > 0 ? max(0, pos0 - p.window + 1) : 0;
     const int first_page = tile_lo / TQK_PAGE;
     w.last_page = (pos0 + count - 1) / TQK_PAGE;
@@ -410,7 +425,7 @@ void attention_prefill_kernel(const PrefillArgs p) {
             page_next = __builtin_amdgcn_readfirstlane(__shfl(my_pages, ahead, TQK_WAVE));
             fetch_page<D>(w, page_next, kr, vr);
         }
-        page_step<D, SPLIT>(w, pg, page_now, kb + cur * L::K_BYTES, vb + cur * L::V_BYTES);
+        page_step<D, SPLIT, CAP>(w, pg, page_now, kb + cur * L::K_BYTES, vb + cur * L::V_BYTES);
         if (pg < w.last_page) stage_page<D>(w, kr, vr, kb + (cur ^ 1) * L::K_BYTES, vb + (cur ^ 1) * L::V_BYTES);
         page_now = page_next;
         ++pg;
@@ -522,12 +537,13 @@ extern "C" int tqk_attention_prefill_tile(int n_tokens, int n_heads, int n_kv_he
     return n_rep == 4 ? 32 : 16;
 }
 
-extern "C" int tqk_attention_prefill(const void* q, const void* keys, const void* values, const int32_t* tok_pos,
-                                     const int32_t* page_table, int table_width, int n_seqs, int n_pages,
-                                     const int32_t* tile_seq, const int32_t* tile_tok0, const int32_t* tile_count,
-                                     int n_tiles, int tile_queries, const int32_t* seq_start, const int32_t* seq_new,
-                                     int window, float scale, void* out, int n_tokens, int n_heads, int n_kv_heads,
-                                     int head_dim, void* stream) {
+extern "C" int tqk_attention_prefill_capped(const void* q, const void* keys, const void* values, const int32_t* tok_pos,
+                                            const int32_t* page_table, int table_width, int n_seqs, int n_pages,
+                                            const int32_t* tile_seq, const int32_t* tile_tok0, const int32_t* tile_count,
+                                            int n_tiles, int tile_queries, const int32_t* seq_start, const int32_t* seq_new,
+                                            int window, float scale, float cap, void* out, int n_tokens, int n_heads, int n_kv_heads,
+                                            int head_dim, void* stream) {
+    TQK_REQUIRE(cap >= 0.f, "tqk_attention_prefill: negative cap");
     TQK_REQUIRE(q && keys && values && tok_pos && page_table && tile_seq && tile_tok0 && tile_count && seq_start && seq_new && out,
                 "tqk_attention_prefill: null pointer");
     TQK_REQUIRE(n_tokens >= 0 && n_tiles >= 0 && n_heads > 0 && n_kv_heads > 0, "tqk_attention_prefill: bad sizes");
@@ -544,7 +560,7 @@ extern "C" int tqk_attention_prefill(const void* q, const void* keys, const void
     a.q = (const bf16_t*)q; a.keys = (const bf16_t*)keys; a.values = (const bf16_t*)values;
     a.tok_pos = tok_pos; a.page_table = page_table; a.table_width = table_width;
     a.tile_seq = tile_seq; a.tile_tok0 = tile_tok0; a.tile_count = tile_count;
-    a.seq_start = seq_start; a.seq_new = seq_new; a.window = window; a.scale = scale;
+    a.seq_start = seq_start; a.seq_new = seq_new; a.window = window; a.scale = scale; a.cap = cap;
     a.out = (bf16_t*)out; a.n_heads = n_heads; a.n_kv_heads = n_kv_heads; a.n_tiles = n_tiles;
     a.tq_shift = tile_queries == 16 ? 4 : (tile_queries == 32 ? 5 : (tile_queries == 64 ? 6 : 7));
     prefill_heads(n_heads / n_kv_heads, tile_queries, &a.heads_per_block, &a.head_chunks);
@@ -566,8 +582,10 @@ extern "C" int tqk_attention_prefill(const void* q, const void* keys, const void
     a.snake_width = (total > n_cus && total <= (long long)per_cu * n_cus) ? n_cus : 0;
     hipStream_t s = (hipStream_t)stream;
     dim3 grid((unsigned)total);
-#define LAUNCH(DD) do { if (split) attention_prefill_kernel<DD, 2><<<grid, waves * TQK_WAVE, 0, s>>>(a); \
-                        else attention_prefill_kernel<DD, 1><<<grid, waves * TQK_WAVE, 0, s>>>(a); } while (0)
+#define LAUNCH(DD) do { if (cap > 0.f) { if (split) attention_prefill_kernel<DD, 2, true><<<grid, waves * TQK_WAVE, 0, s>>>(a); \
+                                         else attention_prefill_kernel<DD, 1, true><<<grid, waves * TQK_WAVE, 0, s>>>(a); } \
+                        else if (split) attention_prefill_kernel<DD, 2, false><<<grid, waves * TQK_WAVE, 0, s>>>(a); \
+                        else attention_prefill_kernel<DD, 1, false><<<grid, waves * TQK_WAVE, 0, s>>>(a); } while (0)
     switch (head_dim) {
         case 32: LAUNCH(32); break;
         case 64: LAUNCH(64); break;
@@ -576,4 +594,14 @@ extern "C" int tqk_attention_prefill(const void* q, const void* keys, const void
     }
 #undef LAUNCH
     return tqk_check_launch("tqk_attention_prefill");
+}
+
+extern "C" int tqk_attention_prefill(const void* q, const void* keys, const void* values, const int32_t* tok_pos,
+                                     const int32_t* page_table, int table_width, int n_seqs, int n_pages,
+                                     const int32_t* tile_seq, const int32_t* tile_tok0, const int32_t* tile_count,
+                                     int n_tiles, int tile_queries, const int32_t* seq_start, const int32_t* seq_new,
+                                     int window, float scale, void* out, int n_tokens, int n_heads, int n_kv_heads,
+                                     int head_dim, void* stream) {
+    return tqk_attention_prefill_capped(q, keys, values, tok_pos, page_table, table_width, n_seqs, n_pages, tile_seq, tile_tok0, tile_count, n_tiles,
+                                        tile_queries, seq_start, seq_new, window, scale, 0.f, out, n_tokens, n_heads, n_kv_heads, head_dim, stream);
 }

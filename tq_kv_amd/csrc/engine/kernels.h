@@ -47,6 +47,8 @@ TQ_QUERY(int, attention_prefill_supported, int);
 TQ_QUERY(int, attention_prefill_tile, int, int, int, int);
 TQ_KERNEL(attention_prefill, cptr, cptr, cptr, ci32, ci32, int, int, int, ci32, ci32, ci32, int, int, ci32, ci32, int, float, void*, int, int,
           int, int, void*);
+TQ_KERNEL(attention_prefill_capped, cptr, cptr, cptr, ci32, ci32, int, int, int, ci32, ci32, ci32, int, int, ci32, ci32, int, float, float, void*, int,
+          int, int, int, void*);
 TQ_KERNEL(swiglu, cptr, void*, int, int, int, void*);
 TQ_KERNEL(gated_act, cptr, void*, int, int, int, int, float, float, void*);
 TQ_KERNEL(fused_gated_act, cptr, cf32, int, float, cptr, int, void*, int, int, int, int, float, float, void*);
@@ -86,6 +88,8 @@ TQ_QUERY(int, ssm_max_state);
 TQ_KERNEL(conv_state, cptr, int, long long, cf32, cf32, cf32, int, int, cf32, long long, ci32, ci32, ci32, ci32, float*, int, int, void*);
 TQ_KERNEL(conv_state_update, cptr, int, long long, cf32, int, float*, long long, ci32, ci32, ci32, int, int, void*);
 TQ_KERNEL(rglru_gates, cf32, cf32, cf32, cf32, cf32, cf32, float*, float*, int, int, int, void*);
+TQ_KERNEL(rglru_gates_any_order, cf32, cf32, cf32, cf32, cf32, cf32, float*, float*, int, int, int, void*);
+TQ_KERNEL(conv_state_step, cptr, int, long long, cf32, cf32, cf32, int, int, float*, long long, ci32, ci32, float*, int, int, void*);
 TQ_KERNEL(linear_scan, cf32, cf32, cptr, int, long long, cf32, float*, long long, ci32, ci32, ci32, void*, int, int, void*);
 TQ_KERNEL(ssm_scan, cf32, long long, cptr, int, long long, cf32, cf32, cf32, float*, long long, ci32, ci32, ci32, float*, int, int, int, int, int, void*);
 TQ_KERNEL(linear_chunks, cf32, cf32, cptr, int, long long, cf32, ci32, ci32, int, float*, float*, void*, int, int, void*);

@@ -516,6 +516,17 @@ private:
                                          n_kv_heads_, head_dim_, value_dim_, c.stream);
                 return;
             }
+            // keys and values of one size, every earlier position visible (or a plain window), no sink: the prompt kernel of the
+            // plain attention takes the cap as an option
+            if (!rows && policy().prefill_mfma && value_dim_ == head_dim_ && keep_first_ == 0 && !sink_ &&
+                K::attention_prefill_supported.raw(head_dim_)) {
+                const int tile = tile_for(c);
+                const Tiles t = last_rows ? c.last_tiles(tile) : c.query_tiles(tile);
+                K::attention_prefill_capped(q.data, entry.keys.data, entry.values.data, tok_pos, table.dev, table.width, c.n_seqs, n_pages, t.seq, t.tok0,
+                                            t.count, t.n, tile, c.dev.seq_start, c.dev.seq_new, window_, scale_, cap_, out.data, n, n_heads_, n_kv_heads_,
+                                            head_dim_, c.stream);
+                return;
+            }
             if (!rows && policy().prefill_mfma) {
                 const int tile = K::attention_masked_mfma_tile.raw(n, n_heads_, n_kv_heads_, head_dim_, value_dim_);
                 const Tiles t = last_rows ? c.last_tiles(tile) : c.query_tiles(tile);

@@ -157,12 +157,19 @@ public:
         float* state = (float*)entry.state.data;
         const Tensor yx = linear(c, x.x, w_yx_, nullptr, dtype).t;
         Tensor u = c.alloc(F32, {n, width_}), a = c.alloc(F32, {n, width_}), g = c.alloc(F32, {n, width_});
-        K::conv_state(at(yx, width_), dtype, 2 * width_, (const float*)x_bias_->t.data, (const float*)conv_w_->t.data, (const float*)conv_b_->t.data, taps_, 0,
-                      state, row, c.dev.tok_seq, c.dev.tok_pos, c.dev.seq_slot, c.dev.seq_start, (float*)u.data, (int)n, (int)width_, c.stream);
-        K::conv_state_update(at(yx, width_), dtype, 2 * width_, (const float*)x_bias_->t.data, taps_, state, row, c.dev.cu, c.dev.seq_new, c.dev.seq_slot,
-                             c.n_seqs, (int)width_, c.stream);
-        K::rglru_gates((const float*)u.data, (const float*)gate_a_->t.data, (const float*)gate_i_->t.data, (const float*)gate_a_b_->t.data,
-                       (const float*)gate_i_b_->t.data, (const float*)decay_c_->t.data, (float*)a.data, (float*)g.data, (int)n, (int)width_, blocks_, c.stream);
+        if (c.all_decode) {
+            K::conv_state_step(at(yx, width_), dtype, 2 * width_, (const float*)x_bias_->t.data, (const float*)conv_w_->t.data, (const float*)conv_b_->t.data,
+                               taps_, 0, state, row, c.dev.tok_seq, c.dev.seq_slot, (float*)u.data, (int)n, (int)width_, c.stream);
+        } else {
+            K::conv_state(at(yx, width_), dtype, 2 * width_, (const float*)x_bias_->t.data, (const float*)conv_w_->t.data, (const float*)conv_b_->t.data, taps_, 0,
+                          state, row, c.dev.tok_seq, c.dev.tok_pos, c.dev.seq_slot, c.dev.seq_start, (float*)u.data, (int)n, (int)width_, c.stream);
+            K::conv_state_update(at(yx, width_), dtype, 2 * width_, (const float*)x_bias_->t.data, taps_, state, row, c.dev.cu, c.dev.seq_new, c.dev.seq_slot,
+                                 c.n_seqs, (int)width_, c.stream);
+        }
+        // (32-bit steps keep one order of the gates' sums whatever the step holds)
+        (dtype == BF16 ? K::rglru_gates_any_order : K::rglru_gates)(
+            (const float*)u.data, (const float*)gate_a_->t.data, (const float*)gate_i_->t.data, (const float*)gate_a_b_->t.data,
+            (const float*)gate_i_b_->t.data, (const float*)decay_c_->t.data, (float*)a.data, (float*)g.data, (int)n, (int)width_, blocks_, c.stream);
         Tensor out = c.alloc(dtype, {n, width_});
         if (in_chunks(c, dtype)) {
             const Chunks ch = c.chunks(SCAN_CHUNK);
@@ -272,10 +279,15 @@ public:
         float* state = (float*)entry.state.data;
         const Tensor zxbcdt = linear(c, x.x, w_in_, nullptr, dtype).t;          // [z | x | B | C | dt | padding]
         Tensor xbc = c.alloc(F32, {n, conv_ch_}), y = c.alloc(F32, {n, inner_});
-        K::conv_state(at(zxbcdt, inner_), dtype, row_, nullptr, (const float*)conv_w_->t.data, (const float*)conv_b_->t.data, taps_, 1, state, row,
-                      c.dev.tok_seq, c.dev.tok_pos, c.dev.seq_slot, c.dev.seq_start, (float*)xbc.data, (int)n, (int)conv_ch_, c.stream);
-        K::conv_state_update(at(zxbcdt, inner_), dtype, row_, nullptr, taps_, state, row, c.dev.cu, c.dev.seq_new, c.dev.seq_slot, c.n_seqs, (int)conv_ch_,
-                             c.stream);
+        if (c.all_decode) {
+            K::conv_state_step(at(zxbcdt, inner_), dtype, row_, nullptr, (const float*)conv_w_->t.data, (const float*)conv_b_->t.data, taps_, 1, state, row,
+                               c.dev.tok_seq, c.dev.seq_slot, (float*)xbc.data, (int)n, (int)conv_ch_, c.stream);
+        } else {
+            K::conv_state(at(zxbcdt, inner_), dtype, row_, nullptr, (const float*)conv_w_->t.data, (const float*)conv_b_->t.data, taps_, 1, state, row,
+                          c.dev.tok_seq, c.dev.tok_pos, c.dev.seq_slot, c.dev.seq_start, (float*)xbc.data, (int)n, (int)conv_ch_, c.stream);
+            K::conv_state_update(at(zxbcdt, inner_), dtype, row_, nullptr, taps_, state, row, c.dev.cu, c.dev.seq_new, c.dev.seq_slot, c.n_seqs, (int)conv_ch_,
+                                 c.stream);
+        }
         if (in_chunks(c, dtype)) {
             const Chunks ch = c.chunks(SCAN_CHUNK);
             const int64_t per_head = (int64_t)n_state_ * p_dim_;

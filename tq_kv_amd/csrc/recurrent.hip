@@ -47,6 +47,86 @@ void conv_state_kernel(const TA* __restrict__ x, long long x_stride, const float
     out[(size_t)t * channels + c] = acc;
 }
 
+// Four values of a row at an aligned place
+__device__ __forceinline__ void load4(const float* p, float (&v)[4]) {
+    const float4 f = *reinterpret_cast<const float4*>(p);
+    v[0] = f.x; v[1] = f.y; v[2] = f.z; v[3] = f.w;
+}
+__device__ __forceinline__ void load4(const bf16_t* p, float (&v)[4]) {
+    const uint2 h = *reinterpret_cast<const uint2*>(p);
+    v[0] = __uint_as_float(h.x << 16); v[1] = __uint_as_float(h.x & 0xffff0000u);
+    v[2] = __uint_as_float(h.y << 16); v[3] = __uint_as_float(h.y & 0xffff0000u);
+}
+
+// The same for steps of many rows: a thread takes four neighbouring channels of CONV_ROWS consecutive rows, reads every
+// input once (the rows' window of CONV_ROWS + TAPS - 1 inputs stays in registers) and the four channels together.  A tap
+// that reaches back before the step's first token of its sequence reads the state instead, as above, and the sum over
+// the taps runs in the same order.
+#define CONV_ROWS 8
+template <typename TA, int TAPS>
+__global__ __launch_bounds__(128)
+void conv_state_vec_kernel(const TA* __restrict__ x, long long x_stride, const float* __restrict__ in_bias, const float* __restrict__ w,
+                           const float* __restrict__ bias, int activation, const float* __restrict__ state, long long state_stride,
+                           const int32_t* __restrict__ tok_seq, const int32_t* __restrict__ tok_pos, const int32_t* __restrict__ seq_slot,
+                           const int32_t* __restrict__ seq_start, float* __restrict__ out, int n_tokens, int channels) {
+    const int c = (blockIdx.x * blockDim.x + threadIdx.x) * 4;
+    if (c >= channels) return;
+    const int t0 = blockIdx.y * CONV_ROWS;
+    float wv[4][TAPS], ib[4], bv[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+#pragma unroll
+        for (int k = 0; k < TAPS; ++k) wv[j][k] = w[(size_t)(c + j) * TAPS + k];
+        ib[j] = in_bias ? in_bias[c + j] : 0.f;
+        bv[j] = bias ? bias[c + j] : 0.f;
+    }
+    float in[CONV_ROWS + TAPS - 1][4];
+#pragma unroll
+    for (int r = 0; r < CONV_ROWS + TAPS - 1; ++r) {
+        const int t = t0 + r - (TAPS - 1);
+        if (t >= 0 && t < n_tokens) {
+            load4(x + (size_t)t * x_stride + c, in[r]);
+#pragma unroll
+            for (int j = 0; j < 4; ++j) in[r][j] += ib[j];
+        } else {
+#pragma unroll
+            for (int j = 0; j < 4; ++j) in[r][j] = 0.f;
+        }
+    }
+#pragma unroll
+    for (int r = 0; r < CONV_ROWS; ++r) {
+        const int t = t0 + r;
+        if (t < n_tokens) {
+            const int seq = tok_seq[t];
+            const int jpos = tok_pos[t] - seq_start[seq];
+            float acc[4] = {0.f, 0.f, 0.f, 0.f};
+            if (jpos >= TAPS - 1) {
+#pragma unroll
+                for (int k = 0; k < TAPS; ++k)
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) acc[j] = fmaf(wv[j][k], in[r + k][j], acc[j]);
+            } else {
+                const float* st = state + (size_t)seq_slot[seq] * state_stride + c;
+#pragma unroll
+                for (int k = 0; k < TAPS; ++k) {
+                    const int back = TAPS - 1 - k;
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) {
+                        const float v = jpos - back >= 0 ? in[r + k][j] : st[(size_t)(TAPS - 1 + jpos - back) * channels + j];
+                        acc[j] = fmaf(wv[j][k], v, acc[j]);
+                    }
+                }
+            }
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                acc[j] += bv[j];
+                if (activation == 1) acc[j] = silu_f(acc[j]);
+            }
+            *reinterpret_cast<float4*>(out + (size_t)t * channels + c) = make_float4(acc[0], acc[1], acc[2], acc[3]);
+        }
+    }
+}
+
 // The state after the step: the last taps - 1 inputs of each sequence, from the step's rows or, where the step brought
 // fewer, from the state before.  A thread per (sequence, channel) reads all it needs before it writes.
 template <typename TA>
@@ -76,52 +156,113 @@ void conv_state_update_kernel(const TA* __restrict__ x, long long x_stride, cons
     }
 }
 
+// Steps of one token a sequence: output and new state in one launch.  A thread per (token, channel) reads the state's
+// taps - 1 inputs, sums in the order of the kernels above, and writes the state moved on by its token's input.
+template <typename TA>
+__global__ __launch_bounds__(256)
+void conv_state_step_kernel(const TA* __restrict__ x, long long x_stride, const float* __restrict__ in_bias, const float* __restrict__ w,
+                            const float* __restrict__ bias, int taps, int activation, float* __restrict__ state, long long state_stride,
+                            const int32_t* __restrict__ tok_seq, const int32_t* __restrict__ seq_slot, float* __restrict__ out, int channels) {
+    const int t = blockIdx.y;
+    const int c = blockIdx.x * blockDim.x + threadIdx.x;
+    if (c >= channels) return;
+    float* st = state + (size_t)seq_slot[tok_seq[t]] * state_stride + c;
+    const float v_new = to_float(x[(size_t)t * x_stride + c]) + (in_bias ? in_bias[c] : 0.f);
+    const int keep = taps - 1;
+    float held[TQK_CONV_MAX_TAPS - 1];
+#pragma unroll
+    for (int i = 0; i < TQK_CONV_MAX_TAPS - 1; ++i) held[i] = i < keep ? st[(size_t)i * channels] : 0.f;
+    float acc = 0.f;
+#pragma unroll
+    for (int i = 0; i < TQK_CONV_MAX_TAPS - 1; ++i)
+        if (i < keep) acc = fmaf(w[(size_t)c * taps + i], held[i], acc);
+    acc = fmaf(w[(size_t)c * taps + keep], v_new, acc);
+    acc += bias ? bias[c] : 0.f;
+    if (activation == 1) acc = silu_f(acc);
+    out[(size_t)t * channels + c] = acc;
+#pragma unroll
+    for (int i = 0; i < TQK_CONV_MAX_TAPS - 1; ++i)
+        if (i < keep) st[(size_t)i * channels] = i + 1 < keep ? held[i + 1 < TQK_CONV_MAX_TAPS - 1 ? i + 1 : i] : v_new;
+}
+
 // ---- gates of the RG-LRU ---------------------------------------------------------------------------------
 // The two gates' matrices are block-diagonal: `blocks` square matrices of bs = width / blocks.  wa_t and wi_t hold them
 // with the input index first, [blocks][bs in][bs out], so that neighbouring threads read neighbouring outputs.  A block
-// of threads takes RG_TOKENS tokens, one diagonal block and up to 256 of its outputs; the tokens' inputs wait in LDS.
-// The sum over the inputs runs in their order, whatever else the step holds.
+// of threads takes RG_TOKENS tokens and one diagonal block; the tokens' inputs wait in LDS, [bs][RG_TOKENS], so that a
+// thread reads an input of all the tokens in two pieces of 16 bytes.
+// KS = 1: a thread per output, up to 256 of them a block; the sum over the inputs runs in their order, whatever else the
+// step holds.  KS = RG_TOKENS: steps of few tokens, where that would leave a few waves walking all the inputs one after
+// the other: a block takes 256 / KS outputs, the inputs are dealt out to KS slices of threads, the slices' sums meet in
+// LDS, and slice k finishes token k.
 #define RG_TOKENS 8
+template <int KS>
 __global__ __launch_bounds__(256)
 void rglru_gates_kernel(const float* __restrict__ u, const float* __restrict__ wa_t, const float* __restrict__ wi_t, const float* __restrict__ ba,
                         const float* __restrict__ bi, const float* __restrict__ decay_c, float* __restrict__ a_out, float* __restrict__ g_out,
                         int n_tokens, int width, int bs) {
-    extern __shared__ float u_lds[];                  // [RG_TOKENS][bs]
+    static_assert(KS == 1 || KS == RG_TOKENS, "a slice finishes a token");
+    extern __shared__ __align__(16) float u_lds[];    // [bs][RG_TOKENS], then (KS > 1) the slices' sums [KS][2][RG_TOKENS][outputs]
     const int t0 = blockIdx.x * RG_TOKENS, b = blockIdx.y;
-    const int o = blockIdx.z * blockDim.x + threadIdx.x;
+    const int outs = blockDim.x / KS;
+    const int slice = threadIdx.x / outs, ol = threadIdx.x % outs;
+    const int o = blockIdx.z * outs + ol;
     const int n_t = min(RG_TOKENS, n_tokens - t0);
     for (int e = threadIdx.x; e < RG_TOKENS * bs; e += blockDim.x) {
         const int k = e / bs, i = e % bs;
-        u_lds[e] = k < n_t ? u[(size_t)(t0 + k) * width + (size_t)b * bs + i] : 0.f;
+        u_lds[i * RG_TOKENS + k] = k < n_t ? u[(size_t)(t0 + k) * width + (size_t)b * bs + i] : 0.f;
     }
     __syncthreads();
-    if (o >= bs) return;
+    if (KS == 1 && o >= bs) return;
     float acc_a[RG_TOKENS], acc_i[RG_TOKENS];
 #pragma unroll
     for (int k = 0; k < RG_TOKENS; ++k) { acc_a[k] = 0.f; acc_i[k] = 0.f; }
-    const float* wa = wa_t + (size_t)b * bs * bs + o;
-    const float* wi = wi_t + (size_t)b * bs * bs + o;
-    for (int i = 0; i < bs; ++i) {
-        const float va = wa[(size_t)i * bs], vi = wi[(size_t)i * bs];
+    const int per = (bs + KS - 1) / KS;
+    const int i0 = slice * per, i1 = min(bs, i0 + per);
+    if (o < bs) {
+        const float* wa = wa_t + (size_t)b * bs * bs + o;
+        const float* wi = wi_t + (size_t)b * bs * bs + o;
+#pragma unroll 4
+        for (int i = i0; i < i1; ++i) {
+            const float va = wa[(size_t)i * bs], vi = wi[(size_t)i * bs];
+            const float4 u0 = *reinterpret_cast<const float4*>(u_lds + i * RG_TOKENS), u1 = *reinterpret_cast<const float4*>(u_lds + i * RG_TOKENS + 4);
+            const float uv[RG_TOKENS] = {u0.x, u0.y, u0.z, u0.w, u1.x, u1.y, u1.z, u1.w};
+#pragma unroll
+            for (int k = 0; k < RG_TOKENS; ++k) {
+                acc_a[k] = fmaf(va, uv[k], acc_a[k]);
+                acc_i[k] = fmaf(vi, uv[k], acc_i[k]);
+            }
+        }
+    }
+    if (KS > 1) {
+        float* red = u_lds + (size_t)bs * RG_TOKENS;
 #pragma unroll
         for (int k = 0; k < RG_TOKENS; ++k) {
-            const float uv = u_lds[k * bs + i];
-            acc_a[k] = fmaf(va, uv, acc_a[k]);
-            acc_i[k] = fmaf(vi, uv, acc_i[k]);
+            red[((slice * 2 + 0) * RG_TOKENS + k) * outs + ol] = acc_a[k];
+            red[((slice * 2 + 1) * RG_TOKENS + k) * outs + ol] = acc_i[k];
         }
+        __syncthreads();
+        if (o >= bs || slice >= n_t) return;
+        float sa = 0.f, si = 0.f;
+#pragma unroll
+        for (int s = 0; s < KS; ++s) {
+            sa += red[((s * 2 + 0) * RG_TOKENS + slice) * outs + ol];
+            si += red[((s * 2 + 1) * RG_TOKENS + slice) * outs + ol];
+        }
+        acc_a[0] = sa; acc_i[0] = si;
     }
     const int ch = b * bs + o;
     const float c8 = decay_c[ch], bav = ba[ch], biv = bi[ch];
 #pragma unroll
-    for (int k = 0; k < RG_TOKENS; ++k) {
+    for (int kk = 0; kk < (KS > 1 ? 1 : RG_TOKENS); ++kk) {
+        const int k = KS > 1 ? slice : kk;
         if (k >= n_t) break;
-        const float r = sigmoid_f(acc_a[k] + bav), gate = sigmoid_f(acc_i[k] + biv);
+        const float r = sigmoid_f(acc_a[kk] + bav), gate = sigmoid_f(acc_i[kk] + biv);
         const float log_a = c8 * r;
         const float a = expf(log_a);
         const float mult = sqrtf(fmaxf(-expm1f(2.f * log_a), 0.f));          // sqrt(1 - a^2), formed without the difference of near-equal numbers
         const size_t at = (size_t)(t0 + k) * width + ch;
         a_out[at] = a;
-        g_out[at] = mult * gate * u_lds[k * bs + o];
+        g_out[at] = mult * gate * u_lds[o * RG_TOKENS + k];
     }
 }
 
@@ -394,6 +535,57 @@ void gated_part_norm_kernel(const float* __restrict__ y, const TA* __restrict__ 
     }
 }
 
+__device__ __forceinline__ void store4(float* p, const float (&v)[4]) { *reinterpret_cast<float4*>(p) = make_float4(v[0], v[1], v[2], v[3]); }
+__device__ __forceinline__ void store4(bf16_t* p, const float (&v)[4]) {
+    uint2 h;
+    h.x = (uint32_t)float_to_bf16_bits(v[0]) | ((uint32_t)float_to_bf16_bits(v[1]) << 16);
+    h.y = (uint32_t)float_to_bf16_bits(v[2]) | ((uint32_t)float_to_bf16_bits(v[3]) << 16);
+    *reinterpret_cast<uint2*>(p) = h;
+}
+
+// The same where a part falls into aligned pieces of four values and a block's threads hold all of it: every value is read and
+// gated once and waits in registers for the part's sum.
+template <typename TA, int ITERS>
+__global__ __launch_bounds__(1024)
+void gated_part_norm_vec_kernel(const float* __restrict__ y, const TA* __restrict__ z, long long z_stride, const float* __restrict__ w, float eps,
+                                TA* __restrict__ out, int size, int part) {
+    __shared__ float scratch[16];
+    const int t = blockIdx.x, g = blockIdx.y;
+    const float* yr = y + (size_t)t * size + (size_t)g * part;
+    const TA* zr = z + (size_t)t * z_stride + (size_t)g * part;
+    float v[ITERS][4];
+    float ss = 0.f;
+#pragma unroll
+    for (int it = 0; it < ITERS; ++it) {
+        const int i = (it * blockDim.x + threadIdx.x) * 4;
+        if (i < part) {
+            float a[4], b[4];
+            load4(yr + i, a);
+            load4(zr + i, b);
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                v[it][j] = a[j] * silu_f(b[j]);
+                ss = fmaf(v[it][j], v[it][j], ss);
+            }
+        } else {
+#pragma unroll
+            for (int j = 0; j < 4; ++j) v[it][j] = 0.f;
+        }
+    }
+    const float inv = 1.f / sqrtf(block_sum(ss, scratch) / (float)part + eps);
+#pragma unroll
+    for (int it = 0; it < ITERS; ++it) {
+        const int i = (it * blockDim.x + threadIdx.x) * 4;
+        if (i < part) {
+            float wv[4], o[4];
+            load4(w + (size_t)g * part + i, wv);
+#pragma unroll
+            for (int j = 0; j < 4; ++j) o[j] = v[it][j] * inv * wv[j];
+            store4(out + (size_t)t * size + (size_t)g * part + i, o);
+        }
+    }
+}
+
 // h += x, float32, element by element
 __global__ __launch_bounds__(256)
 void add_rows_kernel(float* __restrict__ h, const float* __restrict__ x, long long n) {
@@ -415,6 +607,21 @@ extern "C" int tqk_conv_state(const void* x, int x_dtype, long long x_stride, co
     TQK_REQUIRE(activation == 0 || activation == 1, "tqk_conv_state: unknown activation %d", activation);
     if (n_tokens == 0) return 0;
     hipStream_t s = (hipStream_t)stream;
+    // steps of many rows whose rows fall into aligned pieces of four values: the kernel that keeps a window of rows in registers
+    const size_t piece = 4 * (x_dtype == TQK_F32 ? 4 : 2);
+    if (n_tokens >= 2 * CONV_ROWS && (x_dtype == TQK_F32 || x_dtype == TQK_BF16) && channels % 4 == 0 && x_stride % 4 == 0 &&
+        (uintptr_t)x % piece == 0 && (uintptr_t)out % 16 == 0 && (n_tokens + CONV_ROWS - 1) / CONV_ROWS <= 65535) {
+        dim3 grid((channels / 4 + 127) / 128, (n_tokens + CONV_ROWS - 1) / CONV_ROWS);
+#define TQK_CONV(TA, TAPS) conv_state_vec_kernel<TA, TAPS><<<grid, 128, 0, s>>>((const TA*)x, x_stride, in_bias, w, bias, activation, state, state_stride, \
+        tok_seq, tok_pos, seq_slot, seq_start, out, n_tokens, channels)
+#define TQK_CONV_BY_TAPS(TA) switch (taps) { case 1: TQK_CONV(TA, 1); break; case 2: TQK_CONV(TA, 2); break; case 3: TQK_CONV(TA, 3); break; \
+        case 4: TQK_CONV(TA, 4); break; case 5: TQK_CONV(TA, 5); break; case 6: TQK_CONV(TA, 6); break; case 7: TQK_CONV(TA, 7); break; \
+        default: TQK_CONV(TA, 8); break; }
+        if (x_dtype == TQK_F32) TQK_CONV_BY_TAPS(float) else TQK_CONV_BY_TAPS(bf16_t)
+#undef TQK_CONV_BY_TAPS
+#undef TQK_CONV
+        return tqk_check_launch("tqk_conv_state");
+    }
     // (the grid's second dimension takes 65535: longer steps go in pieces)
     for (int t0 = 0; t0 < n_tokens; t0 += 65535) {
         const int n = n_tokens - t0 < 65535 ? n_tokens - t0 : 65535;
@@ -446,19 +653,58 @@ extern "C" int tqk_conv_state_update(const void* x, int x_dtype, long long x_str
     return tqk_check_launch("tqk_conv_state_update");
 }
 
-extern "C" int tqk_rglru_gates(const float* u, const float* wa_t, const float* wi_t, const float* ba, const float* bi, const float* decay_c, float* a_out,
-                               float* g_out, int n_tokens, int width, int blocks, void* stream) {
+extern "C" int tqk_conv_state_step(const void* x, int x_dtype, long long x_stride, const float* in_bias, const float* w, const float* bias, int taps,
+                                   int activation, float* state, long long state_stride, const int32_t* tok_seq, const int32_t* seq_slot, float* out,
+                                   int n_tokens, int channels, void* stream) {
+    TQK_REQUIRE(x && w && state && tok_seq && seq_slot && out, "tqk_conv_state_step: null pointer");
+    TQK_REQUIRE(taps >= 1 && taps <= TQK_CONV_MAX_TAPS, "tqk_conv_state_step: %d taps, the kernel takes 1 to %d", taps, TQK_CONV_MAX_TAPS);
+    TQK_REQUIRE(n_tokens >= 0 && n_tokens <= 65535 && channels > 0 && x_stride >= channels && state_stride >= (long long)(taps - 1) * channels,
+                "tqk_conv_state_step: bad sizes");
+    TQK_REQUIRE(activation == 0 || activation == 1, "tqk_conv_state_step: unknown activation %d", activation);
+    if (n_tokens == 0) return 0;
+    hipStream_t s = (hipStream_t)stream;
+    dim3 grid((channels + 255) / 256, n_tokens);
+    if (x_dtype == TQK_F32)
+        conv_state_step_kernel<float><<<grid, 256, 0, s>>>((const float*)x, x_stride, in_bias, w, bias, taps, activation, state, state_stride, tok_seq, seq_slot, out, channels);
+    else if (x_dtype == TQK_BF16)
+        conv_state_step_kernel<bf16_t><<<grid, 256, 0, s>>>((const bf16_t*)x, x_stride, in_bias, w, bias, taps, activation, state, state_stride, tok_seq, seq_slot, out, channels);
+    else return tqk_fail("tqk_conv_state_step: unknown dtype %d", x_dtype);
+    return tqk_check_launch("tqk_conv_state_step");
+}
+
+static int rglru_gates_launch(const float* u, const float* wa_t, const float* wi_t, const float* ba, const float* bi, const float* decay_c, float* a_out,
+                              float* g_out, int n_tokens, int width, int blocks, int split, void* stream) {
     TQK_REQUIRE(u && wa_t && wi_t && ba && bi && decay_c && a_out && g_out, "tqk_rglru_gates: null pointer");
     TQK_REQUIRE(n_tokens >= 0 && width > 0 && blocks > 0 && width % blocks == 0, "tqk_rglru_gates: width %d in %d blocks", width, blocks);
     const int bs = width / blocks;
-    const size_t lds = (size_t)RG_TOKENS * bs * sizeof(float);
+    size_t lds = (size_t)RG_TOKENS * bs * sizeof(float);
     TQK_REQUIRE(lds <= 64 * 1024, "tqk_rglru_gates: blocks of %d channels, the kernel takes up to %d", bs, 64 * 1024 / (RG_TOKENS * 4));
     TQK_REQUIRE(blocks <= 65535, "tqk_rglru_gates: too many blocks for the grid");
     if (n_tokens == 0) return 0;
+    const int groups = (n_tokens + RG_TOKENS - 1) / RG_TOKENS;
+    // the inputs dealt out to slices where a thread per output would give the chip less than a wave per SIMD
+    if (split && bs >= 2 * RG_TOKENS && bs <= 1024 && (long long)groups * blocks * ((bs + 63) / 64) < 1024) {
+        const int outs = 256 / RG_TOKENS;
+        lds += (size_t)RG_TOKENS * 2 * RG_TOKENS * outs * sizeof(float);
+        dim3 grid(groups, blocks, (bs + outs - 1) / outs);
+        rglru_gates_kernel<RG_TOKENS><<<grid, 256, lds, (hipStream_t)stream>>>(u, wa_t, wi_t, ba, bi, decay_c, a_out, g_out, n_tokens, width, bs);
+        return tqk_check_launch("tqk_rglru_gates");
+    }
     const int threads = bs >= 256 ? 256 : (bs + 63) / 64 * 64;
-    dim3 grid((n_tokens + RG_TOKENS - 1) / RG_TOKENS, blocks, (bs + threads - 1) / threads);
-    rglru_gates_kernel<<<grid, threads, lds, (hipStream_t)stream>>>(u, wa_t, wi_t, ba, bi, decay_c, a_out, g_out, n_tokens, width, bs);
+    dim3 grid(groups, blocks, (bs + threads - 1) / threads);
+    rglru_gates_kernel<1><<<grid, threads, lds, (hipStream_t)stream>>>(u, wa_t, wi_t, ba, bi, decay_c, a_out, g_out, n_tokens, width, bs);
     return tqk_check_launch("tqk_rglru_gates");
+}
+
+extern "C" int tqk_rglru_gates(const float* u, const float* wa_t, const float* wi_t, const float* ba, const float* bi, const float* decay_c, float* a_out,
+                               float* g_out, int n_tokens, int width, int blocks, void* stream) {
+    return rglru_gates_launch(u, wa_t, wi_t, ba, bi, decay_c, a_out, g_out, n_tokens, width, blocks, 0, stream);
+}
+
+/* The same where the order of the sum over the inputs may depend on the step's size (steps of few tokens deal the inputs out to slices). */
+extern "C" int tqk_rglru_gates_any_order(const float* u, const float* wa_t, const float* wi_t, const float* ba, const float* bi, const float* decay_c,
+                                         float* a_out, float* g_out, int n_tokens, int width, int blocks, void* stream) {
+    return rglru_gates_launch(u, wa_t, wi_t, ba, bi, decay_c, a_out, g_out, n_tokens, width, blocks, 1, stream);
 }
 
 extern "C" int tqk_linear_scan(const float* a, const float* g, const void* y, int act_dtype, long long y_stride, const float* y_bias, float* state,
@@ -576,6 +822,21 @@ extern "C" int tqk_gated_part_norm(const float* y, const void* z, int act_dtype,
     if (n_tokens == 0) return 0;
     hipStream_t s = (hipStream_t)stream;
     dim3 grid(n_tokens, parts);
+    {
+        const int part = size / parts, quads = part / 4;
+        const size_t piece = act_dtype == TQK_F32 ? 16 : 8;
+        const int threads = quads >= 1024 ? 1024 : (quads + 63) / 64 * 64;
+        const int iters = threads > 0 ? (quads + threads - 1) / threads : 0;
+        if ((act_dtype == TQK_F32 || act_dtype == TQK_BF16) && part % 4 == 0 && z_stride % 4 == 0 && iters >= 1 && iters <= 4 &&
+            (((uintptr_t)y | (uintptr_t)w) & 15) == 0 && (((uintptr_t)z | (uintptr_t)out) % piece) == 0) {
+#define TQK_GPN(TA, IT) gated_part_norm_vec_kernel<TA, IT><<<grid, threads, 0, s>>>(y, (const TA*)z, z_stride, w, eps, (TA*)out, size, part)
+#define TQK_GPN_BY_ITERS(TA) do { if (iters == 1) TQK_GPN(TA, 1); else if (iters == 2) TQK_GPN(TA, 2); else TQK_GPN(TA, 4); } while (0)
+            if (act_dtype == TQK_F32) TQK_GPN_BY_ITERS(float); else TQK_GPN_BY_ITERS(bf16_t);
+#undef TQK_GPN_BY_ITERS
+#undef TQK_GPN
+            return tqk_check_launch("tqk_gated_part_norm");
+        }
+    }
     if (act_dtype == TQK_F32) gated_part_norm_kernel<float><<<grid, 256, 0, s>>>(y, (const float*)z, z_stride, w, eps, (float*)out, size, size / parts);
     else if (act_dtype == TQK_BF16) gated_part_norm_kernel<bf16_t><<<grid, 256, 0, s>>>(y, (const bf16_t*)z, z_stride, w, eps, (bf16_t*)out, size, size / parts);
     else return tqk_fail("tqk_gated_part_norm: unknown dtype %d", act_dtype);

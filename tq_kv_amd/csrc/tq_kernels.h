@@ -173,6 +173,13 @@ int tqk_attention_prefill(const void* q, const void* keys, const void* values, c
                           int n_tiles, int tile_queries, const int32_t* seq_start, const int32_t* seq_new,
                           int window, float scale, void* out, int n_tokens, int n_heads, int n_kv_heads,
                           int head_dim, void* stream);
+/* The same with a cap on the scores: cap > 0 makes them cap tanh(scale q.k / cap) before the softmax. */
+int tqk_attention_prefill_capped(const void* q, const void* keys, const void* values, const int32_t* tok_pos,
+                                 const int32_t* page_table, int table_width, int n_seqs, int n_pages,
+                                 const int32_t* tile_seq, const int32_t* tile_tok0, const int32_t* tile_count,
+                                 int n_tiles, int tile_queries, const int32_t* seq_start, const int32_t* seq_new,
+                                 int window, float scale, float cap, void* out, int n_tokens, int n_heads, int n_kv_heads,
+                                 int head_dim, void* stream);
 
 /* out[t, i] = silu(gate_up[t, i]) * gate_up[t, inter + i] */
 int tqk_swiglu(const void* gate_up, void* out, int act_dtype, int n_tokens, int inter, void* stream);
@@ -328,7 +335,8 @@ int tqk_rope_norm_store(const void* qkv, int act_dtype, const void* bias, int bi
  *
  * tqk_conv_state: out[t, c] = act(bias[c] + sum_k w[c, k] in(t - (taps - 1 - k), c)), in = x + in_bias for the step's rows (x: rows x_stride
  * values apart, any float dtype) and the state's [taps - 1][channels] (oldest first) for what came before; activation 0: none, 1: silu.
- * tqk_conv_state_update: the state after the step (call it after every reader of the old one). */
+ * tqk_conv_state_update: the state after the step (call it after every reader of the old one).
+ * tqk_conv_state_step: both in one launch for a step in which every sequence brings one token. */
 #define TQK_CONV_MAX_TAPS 8
 int tqk_conv_max_taps(void);
 int tqk_conv_state(const void* x, int x_dtype, long long x_stride, const float* in_bias, const float* w, const float* bias, int taps,
@@ -336,10 +344,16 @@ int tqk_conv_state(const void* x, int x_dtype, long long x_stride, const float* 
                    const int32_t* seq_slot, const int32_t* seq_start, float* out, int n_tokens, int channels, void* stream);
 int tqk_conv_state_update(const void* x, int x_dtype, long long x_stride, const float* in_bias, int taps, float* state, long long state_stride,
                           const int32_t* cu, const int32_t* seq_new, const int32_t* seq_slot, int n_seqs, int channels, void* stream);
+int tqk_conv_state_step(const void* x, int x_dtype, long long x_stride, const float* in_bias, const float* w, const float* bias, int taps,
+                        int activation, float* state, long long state_stride, const int32_t* tok_seq, const int32_t* seq_slot, float* out,
+                        int n_tokens, int channels, void* stream);
 /* Gates of a real-gated linear recurrent unit: r = sigmoid(Wa u + ba), i = sigmoid(Wi u + bi) with block-diagonal Wa, Wi given as
  * [blocks][in][out]; a = exp(decay_c r) (decay_c = -8 softplus(lam), per channel); g = sqrt(1 - a^2) i u. */
 int tqk_rglru_gates(const float* u, const float* wa_t, const float* wi_t, const float* ba, const float* bi, const float* decay_c, float* a_out,
                     float* g_out, int n_tokens, int width, int blocks, void* stream);
+/* (the same; the order of the sum over the inputs may depend on the step's size: steps of few tokens deal the inputs out to slices of threads) */
+int tqk_rglru_gates_any_order(const float* u, const float* wa_t, const float* wi_t, const float* ba, const float* bi, const float* decay_c,
+                              float* a_out, float* g_out, int n_tokens, int width, int blocks, void* stream);
 /* S_t = a_t S_(t-1) + g_t per sequence and channel from the state (one float a channel), which is left at the last S;
  * out_t = S_t gelu_tanh(y_t + y_bias) in the activation dtype. */
 int tqk_linear_scan(const float* a, const float* g, const void* y, int act_dtype, long long y_stride, const float* y_bias, float* state,
