@@ -55,7 +55,9 @@ def config_odd():
 
 # One layer of one kind and a configuration without a loop.
 def config_single(kind, width=64):
-    mix = {"attention": attention(4, 2, 16, 24, 8, base=50.0, scale=1.0, softcap=30.0), "rglru": rglru(48, 3, 4), "mamba2": mamba2(4, 12, 16, 2, 4, 2)}[kind]
+    # ("attention_equal": keys and values of one size, which the plain prompt kernel takes with the cap as an option)
+    mix = {"attention": attention(4, 2, 16, 24, 8, base=50.0, scale=1.0, softcap=30.0),
+           "attention_equal": attention(6, 2, 32, 32, 12, base=50.0, scale=0.7, softcap=30.0), "rglru": rglru(48, 3, 4), "mamba2": mamba2(4, 12, 16, 2, 4, 2)}[kind]
     return config(97, width, [(mix, 48)], scale=5.0)
 
 

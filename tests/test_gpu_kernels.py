@@ -307,12 +307,14 @@ def paged(k, v, page_ids, n_pages, dtype):
     return keys, values
 
 
-def attention_reference(q, k, v, pos, window, scale):
-    """q [T, nh, d] at absolute positions pos over k, v [nkv, S, d]: plain softmax attention."""
+def attention_reference(q, k, v, pos, window, scale, cap=0.0):
+    """q [T, nh, d] at absolute positions pos over k, v [nkv, S, d]: plain softmax attention (cap > 0: of cap tanh(score / cap))."""
     nh = q.shape[1]
     n_rep = nh // k.shape[0]
     kk, vv = plain.repeat_kv(k, n_rep), plain.repeat_kv(v, n_rep)
     att = torch.einsum("thd,hsd->hts", q, kk) * scale
+    if cap:
+        att = cap * torch.tanh(att / cap)
     j = torch.arange(k.shape[1])[None, :]
     vis = j <= pos[:, None]
     if window:
@@ -714,7 +716,8 @@ def test_attention_decode_refuses_other_head_sizes():
 @pytest.mark.parametrize("nh,nkv,d", [(28, 4, 128), (6, 2, 64), (5, 5, 32), (10, 2, 32), (3, 1, 96), (40, 2, 64), (12, 2, 128)])
 @pytest.mark.parametrize("window", [0, 70, 12])
 @pytest.mark.parametrize("tile", [16, 32, 64, 128])
-def test_attention_prefill(nh, nkv, d, window, tile):
+@pytest.mark.parametrize("cap", [0.0, 4.0])
+def test_attention_prefill(nh, nkv, d, window, tile, cap):
     # sequence 0: 150 new queries at positions 150..299 behind 150 cached ones; sequence 1: a
     # whole prompt of 70; sequence 2: one token at position 0.  Pages scrambled, unread places NaN.
     spans = [(150, 300), (0, 70), (0, 1)]
@@ -747,15 +750,18 @@ def test_attention_prefill(nh, nkv, d, window, tile):
     scale = 1 / math.sqrt(d)
     K.attention_prefill(q, keys, values, pos.to(torch.int32).to(DEV), ints(tables), ints(tile_seq), ints(tile_tok0),
                         ints(tile_count), ints([a for a, _ in spans]), ints([b - a for a, b in spans]), window, scale, out,
-                        tile_queries=tile)
+                        tile_queries=tile, cap=cap)
     off = 0
     for i, (a, b) in enumerate(spans):
-        want = attention_reference(qs[i].float(), ks[i], vs[i], torch.arange(a, b), window, scale)
+        want = attention_reference(qs[i].float(), ks[i], vs[i], torch.arange(a, b), window, scale, cap)
         torch.testing.assert_close(out[off:off + b - a].float().cpu(), want, atol=2e-2, rtol=2e-2)
         off += b - a
-    if window != 70:
+    if window != 70 and not cap:
         other = attention_reference(qs[0][-1:].float(), ks[0], vs[0], torch.tensor([299]), 70, scale)
         assert (other - out[149:150].float().cpu()).abs().max() > 0.1
+    if cap and window != 12:         # the cap matters where a marked key is in sight: their scores lie far above it
+        other = attention_reference(qs[0][-1:].float(), ks[0], vs[0], torch.tensor([299]), window, scale, 0.0)
+        assert (other - out[149:150].float().cpu()).abs().max() > 0.05
 
 
 # ---- skinny products with norm, residual sum, gate and rotation folded in ----------------------

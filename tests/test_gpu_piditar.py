@@ -128,6 +128,7 @@ def test_the_convolution_reads_its_first_inputs_from_the_state_and_zeros_before_
 # ---- whole models ----------------------------------------------------------------------------------------
 _MODELS = {}
 MAKERS = {"mixed": C.config_mixed, "ones": C.config_ones, "odd": C.config_odd, "attention": lambda: C.config_single("attention"),
+          "attention_equal": lambda: C.config_single("attention_equal"),
           "rglru": lambda: C.config_single("rglru"), "mamba2": lambda: C.config_single("mamba2")}
 
 
@@ -242,10 +243,11 @@ def logits_of(eng, tokens, how, n):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-def test_a_token_reaches_every_later_position_through_attention_and_none_before(dtype, tmp_path_factory):
+@pytest.mark.parametrize("name", ["attention", "attention_equal"])
+def test_a_token_reaches_every_later_position_through_attention_and_none_before(name, dtype, tmp_path_factory):
     """One attention layer with a scale that lets single keys carry the output: changing the token at j changes the logits at i if and only
     if j <= i.  Queries in a prompt, in a later portion, and decoded one by one; keys at the sequence's start, at page borders and far away."""
-    cfg, w, eng = engine("attention", dtype, tmp_path_factory)
+    cfg, w, eng = engine(name, dtype, tmp_path_factory)
     n = 200
     toks = C.tokens(n, cfg["vocab"], 8)
     for how in ("prompt", "portions", "decoded"):
@@ -265,11 +267,12 @@ def test_a_token_reaches_every_later_position_through_attention_and_none_before(
                     assert moved == 0.0, "%s: query %d sees the later token at %d" % (how, i, j)
 
 
-def test_one_key_far_away_among_hundreds_carries_the_output(tmp_path_factory):
+@pytest.mark.parametrize("vdim", [24, 64])
+def test_one_key_far_away_among_hundreds_carries_the_output(vdim, tmp_path_factory):
     """Two tokens have an element of the embedding to themselves; the keys of the one and the queries of the other read it with one and the
     same long vector, so that this key's score stands far above three hundred random ones: the output at the query is that token's value,
     wherever the token stands (first, at a page's border, far back) and however the query comes (in the prompt or decoded)."""
-    cfg = C.config(60, 32, [(C.attention(2, 1, 64, 24, 0, scale=1.0, softcap=100.0), None)], scale=1.0)
+    cfg = C.config(60, 32, [(C.attention(2, 1, 64, vdim, 0, scale=1.0, softcap=100.0), None)], scale=1.0)
     n, special, asker = 330, 7, 11
     toks = [t if t not in (special, asker) else 20 for t in C.tokens(n, cfg["vocab"], 2)]
     f = C.as_float(C.weights(cfg, 4))
