@@ -95,6 +95,38 @@ def test_a_mixer_alone(dtype, mix):
             cache.release(s)
 
 
+@pytest.mark.parametrize("style", ["pairs", "halves"])
+@pytest.mark.parametrize("m", [C.attention(6, 2, 64, 40, 24), C.attention(2, 1, 160, 16, 160), C.attention(4, 4, 24, 24, 0)], ids=lambda m: "x".join(str(v) for v in m[1].values() if isinstance(v, int)))
+def test_long_steps_turn_and_norm_heads_as_short_ones_do(style, m):
+    """Steps of more than 64 tokens add the biases, turn and norm the heads in pieces of several elements and store the values with the
+    lanes along the tokens; shorter steps go element by element.  Both orders of rotation, the same tokens either way."""
+    hidden, eps = 72, 1e-5
+    spec = mixer_spec("attention", m[1], hidden, eps)
+    if m[1]["rot"]["dims"]:
+        spec.params["position"].params["style"] = style
+    cfg = C.config(50, hidden, [(m, None)])
+    w = {k[len("l0.mix."):]: v for k, v in C.weights(cfg, 5).items() if k.startswith("l0.mix.")}
+    env = BuildEnv(DEV, torch.bfloat16)
+    part = env.build("mixer", spec)
+    part.load({k: v.to(DEV) for k, v in w.items()})
+    cache = Cache([part.cache_need()], [None], 64 * 8, 2, torch.bfloat16, DEV)
+    x = torch.randn(200, hidden).to(torch.bfloat16)
+    got = []
+    for cuts in ([200], [40, 40, 40, 40, 40]):
+        slot, a, out = cache.acquire(), 0, []
+        for n in cuts:
+            ctx, sizes = step_ctx(cache, [(slot, [0] * n)])
+            out.append(part.forward(x[a:a + n].to(DEV), ctx, cache.entry(0)))
+            cache.commit(sizes)
+            a += n
+        cache.release(slot)
+        got.append(torch.cat(out).float())
+    assert C.row_errors(got[0], got[1]).max().item() < 0.02
+    if style == "pairs":
+        want = plain.mixer("attention", x.float(), C.as_float(w), "", m[1], eps, torch.arange(200), torch.bfloat16)
+        assert C.row_errors(got[0], want).max().item() < 0.02
+
+
 def test_the_convolution_reads_its_first_inputs_from_the_state_and_zeros_before_the_start():
     """One channel group with weights 1, 10, 100, 1000 on the four taps and no recurrence to speak of (the decay is driven to zero): what a token's
     output holds of each earlier input can be read off, whole and in portions of one token."""

@@ -149,6 +149,112 @@ void rope_norm_store_kernel(const TA* __restrict__ qkv, const TB* __restrict__ b
     }
 }
 
+// Steps of many tokens in bfloat16, head sizes multiples of 8, in two launches.  Queries and keys: a wave per head as above, a lane
+// takes VEC neighbouring elements in one load and one store (2 for heads up to 128, else 4); turned in pairs, an element's partner
+// is in the same lane.  Values: the lanes along the tokens, as mixed_values_store_vec_kernel below has them.
+template <typename TB, int VEC>
+__global__ __launch_bounds__(AM_WAVES * TQK_WAVE)
+void rope_norm_qk_vec_kernel(const bf16_t* __restrict__ qkv, const TB* __restrict__ bias, const float* __restrict__ cos_table,
+                             const float* __restrict__ sin_table, int rot_dim, int style, int max_positions, int normed, float eps,
+                             const int32_t* __restrict__ tok_seq, const int32_t* __restrict__ tok_pos, const int32_t* __restrict__ page_table,
+                             int table_width, bf16_t* __restrict__ keys, bf16_t* __restrict__ q_out, int n_heads, int n_kv_heads, int dk, int dv,
+                             int write_kv) {
+    const int t = blockIdx.x;
+    const int head = blockIdx.y * AM_WAVES + threadIdx.x / TQK_WAVE;
+    const int lane = threadIdx.x % TQK_WAVE;
+    if (head >= n_heads + (write_kv ? n_kv_heads : 0)) return;
+    const int pos = tok_pos[t];
+    const bool is_key = head >= n_heads;
+    const size_t total = (size_t)(n_heads + n_kv_heads) * dk + (size_t)n_kv_heads * dv;
+    const bf16_t* row = qkv + (size_t)t * total;
+    int page = -1;
+    if (is_key) {
+        page = page_table[(size_t)tok_seq[t] * table_width + pos / TQK_PAGE];
+        if (page < 0) return;                          // the host never lets this happen
+    }
+    const size_t off = (size_t)head * dk;
+    const int half = rot_dim / 2;
+    const bool rotate = rot_dim > 0 && style != 0 && pos < max_positions;
+    const int i0 = lane * VEC;
+    float x[VEC];
+    float ss = 0.f;
+    if (i0 < dk) {
+        float raw[VEC];
+        if (VEC == 2) {
+            const uint32_t u = *reinterpret_cast<const uint32_t*>(row + off + i0);
+            raw[0] = __uint_as_float(u << 16); raw[1] = __uint_as_float(u & 0xffff0000u);
+        } else {
+            const uint2 u = *reinterpret_cast<const uint2*>(row + off + i0);
+            raw[0] = __uint_as_float(u.x << 16); raw[1] = __uint_as_float(u.x & 0xffff0000u);
+            raw[VEC - 2] = __uint_as_float(u.y << 16); raw[VEC - 1] = __uint_as_float(u.y & 0xffff0000u);
+        }
+        if (bias) {
+#pragma unroll
+            for (int j = 0; j < VEC; ++j) raw[j] += to_float(bias[off + i0 + j]);
+        }
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) {
+            const int i = i0 + j;
+            float v = raw[j];
+            if (rotate && i < rot_dim) {
+                bool first;
+                float y;
+                int p;
+                if (style == 2) {
+                    first = (j & 1) == 0; y = raw[j ^ 1]; p = i / 2;
+                } else {
+                    first = i < half;
+                    const int partner = first ? i + half : i - half;
+                    y = to_float(row[off + partner]) + (bias ? to_float(bias[off + partner]) : 0.f);
+                    p = first ? i : i - half;
+                }
+                const float c = cos_table[(size_t)pos * half + p], sn = sin_table[(size_t)pos * half + p];
+                v = first ? v * c - y * sn : v * c + y * sn;
+            }
+            x[j] = v;
+            ss = fmaf(v, v, ss);
+        }
+    }
+    const float inv = normed ? 1.f / sqrtf(wave_sum(ss) / (float)dk + eps) : 1.f;
+    if (i0 >= dk) return;
+    bf16_t* dst = !is_key ? q_out + ((size_t)t * n_heads + head) * dk
+                          : keys + (((size_t)page * n_kv_heads + (head - n_heads)) * TQK_PAGE + pos % TQK_PAGE) * dk;
+    uint32_t packed[VEC / 2];
+#pragma unroll
+    for (int j = 0; j < VEC / 2; ++j)
+        packed[j] = (uint32_t)float_to_bf16_bits(x[2 * j] * inv) | ((uint32_t)float_to_bf16_bits(x[2 * j + 1] * inv) << 16);
+    if (VEC == 2) *reinterpret_cast<uint32_t*>(dst + i0) = packed[0];
+    else *reinterpret_cast<uint2*>(dst + i0) = make_uint2(packed[0], packed[VEC / 2 - 1]);
+}
+
+template <typename TB>
+__global__ __launch_bounds__(256)
+void biased_values_store_vec_kernel(const bf16_t* __restrict__ qkv, const TB* __restrict__ bias, const int32_t* __restrict__ tok_seq,
+                                    const int32_t* __restrict__ tok_pos, const int32_t* __restrict__ page_table, int table_width,
+                                    bf16_t* __restrict__ values, int n_tokens, int n_heads, int n_kv_heads, int dk, int dv) {
+    const int lane = threadIdx.x % TQK_WAVE, wave = threadIdx.x / TQK_WAVE, n_waves = blockDim.x / TQK_WAVE;
+    const int t = (blockIdx.x / n_kv_heads) * TQK_WAVE + lane, g = blockIdx.x % n_kv_heads;
+    if (t >= n_tokens) return;
+    const int pos = tok_pos[t];
+    const int page = page_table[(size_t)tok_seq[t] * table_width + pos / TQK_PAGE];
+    if (page < 0) return;                               // the host never lets this happen
+    bf16_t* dst = values + ((size_t)page * n_kv_heads + g) * TQK_PAGE * dv + value_place(pos % TQK_PAGE);
+    const size_t total = (size_t)(n_heads + n_kv_heads) * dk + (size_t)n_kv_heads * dv;
+    const size_t off = (size_t)(n_heads + n_kv_heads) * dk + (size_t)g * dv;
+    const bf16_t* src = qkv + (size_t)t * total + off;
+    for (int c = wave * 8; c < dv; c += n_waves * 8) {
+        const uint4 raw = *reinterpret_cast<const uint4*>(src + c);
+        const uint32_t u[4] = {raw.x, raw.y, raw.z, raw.w};
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            float lo = __uint_as_float(u[j] << 16), hi = __uint_as_float(u[j] & 0xffff0000u);
+            if (bias) { lo += to_float(bias[off + c + 2 * j]); hi += to_float(bias[off + c + 2 * j + 1]); }
+            dst[(size_t)(c + 2 * j) * TQK_PAGE].bits = float_to_bf16_bits(lo);
+            dst[(size_t)(c + 2 * j + 1) * TQK_PAGE].bits = float_to_bf16_bits(hi);
+        }
+    }
+}
+
 // The same for steps of many tokens in bfloat16 (head sizes multiples of 8, half the rotated elements too), in two launches.
 // Queries and keys: a block per token, a thread per 8 neighbouring elements (16 bytes a load and a store); the sums of squares of a
 // head's pieces meet in LDS; the piece a rotated one turns with is read once more (it is in the caches).
@@ -414,6 +520,22 @@ extern "C" int tqk_rope_norm_store(const void* qkv, int act_dtype, const void* b
     TQK_REQUIRE(!write_kv || (tok_seq && page_table && keys && values && table_width > 0), "tqk_rope_norm_store: no cache to write to");
     if (n_tokens == 0) return 0;
     hipStream_t s = (hipStream_t)stream;
+    if (act_dtype == TQK_BF16 && n_tokens > 64 && key_dim % 8 == 0 && value_dim % 8 == 0 && (!bias || bias_dtype == TQK_BF16 || bias_dtype == TQK_F32) &&
+        (((uintptr_t)qkv | (uintptr_t)keys | (uintptr_t)q_out) & 15) == 0) {
+        dim3 qk_grid(n_tokens, (n_heads + (write_kv ? n_kv_heads : 0) + AM_WAVES - 1) / AM_WAVES);
+        const long long v_blocks = (long long)((n_tokens + TQK_WAVE - 1) / TQK_WAVE) * n_kv_heads;
+        TQK_REQUIRE(v_blocks <= 0x7fffffff, "tqk_rope_norm_store: too many tokens");
+#define TQK_RNV(TB, VEC) \
+        rope_norm_qk_vec_kernel<TB, VEC><<<qk_grid, AM_WAVES * TQK_WAVE, 0, s>>>((const bf16_t*)qkv, (const TB*)bias, cos_table, sin_table, rot_dim, style, \
+            max_positions, normed, eps, tok_seq, tok_pos, page_table, table_width, (bf16_t*)keys, (bf16_t*)q_out, n_heads, n_kv_heads, key_dim, value_dim, write_kv)
+#define TQK_RNV_ALL(TB) do { if (key_dim <= 128) TQK_RNV(TB, 2); else TQK_RNV(TB, 4); \
+        if (write_kv) biased_values_store_vec_kernel<TB><<<(unsigned)v_blocks, 256, 0, s>>>((const bf16_t*)qkv, (const TB*)bias, tok_seq, tok_pos, page_table, \
+            table_width, (bf16_t*)values, n_tokens, n_heads, n_kv_heads, key_dim, value_dim); } while (0)
+        if (bias && bias_dtype == TQK_F32) TQK_RNV_ALL(float); else TQK_RNV_ALL(bf16_t);
+#undef TQK_RNV_ALL
+#undef TQK_RNV
+        return tqk_check_launch("tqk_rope_norm_store");
+    }
     dim3 grid(n_tokens, (n_heads + 2 * n_kv_heads + AM_WAVES - 1) / AM_WAVES);
 #define TQK_RNS(TA, TB) \
     rope_norm_store_kernel<TA, TB><<<grid, AM_WAVES * TQK_WAVE, 0, s>>>((const TA*)qkv, (const TB*)bias, cos_table, sin_table, rot_dim, style, max_positions, \
