@@ -114,6 +114,13 @@ static void k_fused_store(StepContext& c, const Tensor& x, const int32_t* rows, 
                    out.data, out.dtype, (int)out.shape[0], (int)w.n, (int)w.k, c.stream);
 }
 
+Tensor linear_of_norm(StepContext& c, const LazyNorm& norm, const Weight& w, int out_dtype) {
+    if (!fusable(norm.xw.shape[0], w)) raise(TQE_ERR_STATE, "a folded norm was handed to a product that the few-row kernel does not take");
+    Tensor out = c.alloc(out_dtype, {norm.xw.shape[0], w.n});
+    k_fused_store(c, norm.xw, nullptr, &norm, w, out);
+    return out;
+}
+
 static void k_fused_gated(StepContext& c, const Tensor& x, const LazyNorm* norm, const Weight& w, Tensor& out, const Gate& gate) {
     int packed = 0;
     const void* wp = few_ptr(w, &packed);

@@ -64,6 +64,9 @@ struct Product {
 // x [M, K] times weight^T -> [M, N] of out_dtype (into `out` if given, else workspace memory).
 // leave_sums: the caller also takes the product unfinished where the kernel cuts K into pieces.
 Product linear(StepContext& c, const Tensor& x, const Weight& w, const Tensor* bias, int out_dtype, bool leave_sums = false, Tensor* out = nullptr);
+// The same for a step of few rows whose input is a folded norm: the stream times the norm's weight goes in, and the kernel divides
+// its result by the rows' root mean square (where fusable(rows, w) holds).
+Tensor linear_of_norm(StepContext& c, const LazyNorm& norm, const Weight& w, int out_dtype);
 // Which gate a gated feed-forward applies to its gate and up products g and u (the kernels' TQK_GATE_* codes):
 // silu g sigmoid(g) u; relu max(g, 0) u; clamped g' sigmoid(alpha g') (u' + 1) with g' = min(g, limit) and
 // u' = clamp(u, -limit, limit); gelu gelu_tanh(g) u; relu2 max(g, 0)^2 u.  A feed-forward without a gate product applies the

@@ -394,7 +394,11 @@ public:
         if (tb.style != STYLE_HALVES || tb.rot_dim != head_dim_) return false;
         return !b_qkv_ || b_qkv_->t.dtype == BF16;
     }
-    bool folds_norm(const StepContext& c) const override { return fused_qkv_ok(c) && !reads_other_cache; }
+    bool folds_norm(const StepContext& c) const override {
+        // (with biases first and the heads' norm after the rotation: the product alone divides by the rows' root mean square)
+        if (extras_) return turned_first_ && c.all_decode && fusable(c.n_tokens, w_qkv_) && !reads_other_cache;
+        return fused_qkv_ok(c) && !reads_other_cache;
+    }
     bool adds_to_stream(const StepContext& c) const override {
         return !b_o_ && (fusable(c.n_tokens, w_o_, true) || leaves_sums(c.n_tokens, w_o_));
     }
@@ -407,8 +411,8 @@ public:
         Tensor q = c.alloc(dtype, {n, n_heads_, head_dim_});
         const int n_pages = (int)entry.keys.shape[0];
         if (extras_) {
-            if (x.lazy) raise(TQE_ERR_STATE, "attention: this configuration takes no folded norm");
-            if (turned_first_) turned_qkv(c, x.x, entry, table, q);
+            if (x.lazy && !turned_first_) raise(TQE_ERR_STATE, "attention: this configuration takes no folded norm");
+            if (turned_first_) turned_qkv(c, x, entry, table, q);
             else normed_qkv(c, x.x, entry, table, q);
         } else if (x.lazy || (c.fuse_small && entry.writes && fused_qkv_ok(c))) {
             if (x.lazy && !entry.writes) raise(TQE_ERR_STATE, "a run that reads another run's cache cannot take a folded norm");
@@ -474,9 +478,11 @@ private:
     }
 
     // product, then biases, rotation (halves or pairs), the heads' norm without a weight after it, and the cache write in one kernel
-    void turned_qkv(StepContext& c, const Tensor& x, const CacheEntry& entry, const StepContext::Table& table, Tensor& q) {
-        const int64_t n = x.shape[0];
-        Product p = linear(c, x, w_qkv_, nullptr, x.dtype);
+    void turned_qkv(StepContext& c, const Activation& x, const CacheEntry& entry, const StepContext::Table& table, Tensor& q) {
+        const int64_t n = x.rows();
+        Product p;
+        if (x.lazy) p.t = linear_of_norm(c, x.norm, w_qkv_, BF16);
+        else p = linear(c, x.x, w_qkv_, nullptr, x.x.dtype);
         const Position::Tables tb = position_->tables();
         const bool turn = tb.style != STYLE_NONE;
         const bool write = entry.writes;

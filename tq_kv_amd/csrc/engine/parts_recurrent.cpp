@@ -147,15 +147,17 @@ public:
         return n;
     }
     bool adds_to_stream(const StepContext& c) const override { return fusable(c.n_tokens, w_o_, true) || leaves_sums(c.n_tokens, w_o_); }
+    // (steps of few rows: the first product divides by the rows' root mean square itself)
+    bool folds_norm(const StepContext& c) const override { return fusable(c.n_tokens, w_yx_); }
 
     Tensor forward(StepContext& c, const Activation& x, const CacheEntry& entry, Stream* stream, bool last_rows) override {
         if (entry.kind != CacheNeed::State || !entry.writes) raise(TQE_ERR_STATE, "rglru was given no state of its own in the cache");
-        if (x.lazy || last_rows) raise(TQE_ERR_STATE, "rglru takes the normed step itself, all rows of it");
-        const int64_t n = x.x.shape[0];
-        const int dtype = x.x.dtype;
+        if (last_rows) raise(TQE_ERR_STATE, "rglru takes all rows of the step");
+        const int64_t n = x.rows();
+        const int dtype = x.lazy ? BF16 : x.x.dtype;
         const long long row = entry.state.cols(), conv_part = (long long)(taps_ - 1) * width_;
         float* state = (float*)entry.state.data;
-        const Tensor yx = linear(c, x.x, w_yx_, nullptr, dtype).t;
+        const Tensor yx = x.lazy ? linear_of_norm(c, x.norm, w_yx_, dtype) : linear(c, x.x, w_yx_, nullptr, dtype).t;
         Tensor u = c.alloc(F32, {n, width_}), a = c.alloc(F32, {n, width_}), g = c.alloc(F32, {n, width_});
         if (c.all_decode) {
             K::conv_state_step(at(yx, width_), dtype, 2 * width_, (const float*)x_bias_->t.data, (const float*)conv_w_->t.data, (const float*)conv_b_->t.data,
@@ -269,15 +271,16 @@ public:
         return n;
     }
     bool adds_to_stream(const StepContext& c) const override { return fusable(c.n_tokens, w_o_, true) || leaves_sums(c.n_tokens, w_o_); }
+    bool folds_norm(const StepContext& c) const override { return fusable(c.n_tokens, w_in_); }
 
     Tensor forward(StepContext& c, const Activation& x, const CacheEntry& entry, Stream* stream, bool last_rows) override {
         if (entry.kind != CacheNeed::State || !entry.writes) raise(TQE_ERR_STATE, "mamba2 was given no state of its own in the cache");
-        if (x.lazy || last_rows) raise(TQE_ERR_STATE, "mamba2 takes the normed step itself, all rows of it");
-        const int64_t n = x.x.shape[0];
-        const int dtype = x.x.dtype;
+        if (last_rows) raise(TQE_ERR_STATE, "mamba2 takes all rows of the step");
+        const int64_t n = x.rows();
+        const int dtype = x.lazy ? BF16 : x.x.dtype;
         const long long row = entry.state.cols(), conv_part = (long long)(taps_ - 1) * conv_ch_;
         float* state = (float*)entry.state.data;
-        const Tensor zxbcdt = linear(c, x.x, w_in_, nullptr, dtype).t;          // [z | x | B | C | dt | padding]
+        const Tensor zxbcdt = x.lazy ? linear_of_norm(c, x.norm, w_in_, dtype) : linear(c, x.x, w_in_, nullptr, dtype).t;          // [z | x | B | C | dt | padding]
         Tensor xbc = c.alloc(F32, {n, conv_ch_}), y = c.alloc(F32, {n, inner_});
         if (c.all_decode) {
             K::conv_state_step(at(zxbcdt, inner_), dtype, row_, nullptr, (const float*)conv_w_->t.data, (const float*)conv_b_->t.data, taps_, 1, state, row,
