@@ -38,6 +38,10 @@ class Entry:
 
     def __init__(self, cache, run, group, index, writes):
         self.cache, self.run, self.group, self.writes = cache, run, group, writes
+        self.attach(group, index)
+
+    def attach(self, group, index):
+        """A run may have pages and a state row: the entry shows both (its group is the first it was given)."""
         if isinstance(group, KVGroup):
             self.keys, self.values = group.keys[index], group.values[index]
         else:
@@ -171,7 +175,9 @@ class Cache:
                 continue
             owner = run if cache_of[run] is None else cache_of[run]
             for group in self.kv_groups + self.state_groups:
-                if owner in group.runs:
+                if owner in group.runs and run in self._views:
+                    self._views[run].attach(group, group.runs.index(owner))
+                elif owner in group.runs:
                     self._views[run] = Entry(self, run, group, group.runs.index(owner), cache_of[run] is None)
 
     @classmethod

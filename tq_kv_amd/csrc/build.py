@@ -18,13 +18,13 @@ import time
 
 HERE = os.path.dirname(os.path.abspath(__file__))
 SOURCES = ["host.cpp", "elementwise.hip", "gemm_generic.hip", "attention_generic.hip", "sampling.hip",
-           "attention_decode.hip", "attention_prefill.hip", "skinny_fused.hip", "mid_product.hip", "random_init.hip", "utility.hip", "probe.hip", "latent.hip", "moe.hip", "grouped.hip", "stream_ops.hip", "attention_masked.hip", "attention_masked_mfma.hip", "recurrent.hip"]
+           "attention_decode.hip", "attention_prefill.hip", "skinny_fused.hip", "mid_product.hip", "random_init.hip", "utility.hip", "probe.hip", "latent.hip", "moe.hip", "grouped.hip", "stream_ops.hip", "attention_masked.hip", "attention_masked_mfma.hip", "recurrent.hip", "streams.hip", "linear_attention.hip", "pooled_attention.hip"]
 HEADERS = ["common.h", "tq_kernels.h", "tq_no_alloc.h"]
 # the engine: host code only (config, weights, parts, model, cache, step, loop), built with the host compiler into a
 # library of its own that reaches the GPU through the HIP runtime, hipBLASLt and the kernel library above
 HOST_SOURCES = ["host_engine.cpp"] + ["engine/" + n for n in (
     "api.cpp", "config.cpp", "core.cpp", "engine.cpp", "generate.cpp", "json.cpp", "linear.cpp", "model.cpp", "parts_builtin.cpp",
-    "nikasun.cpp", "sizudra.cpp", "parts_latent.cpp", "parts_moe.cpp", "parts_stream.cpp", "parts_recurrent.cpp", "piditar.cpp", "plugin.cpp", "qwen2.cpp", "spec.cpp", "step.cpp", "store.cpp", "trace.cpp", "weights.cpp")]
+    "nikasun.cpp", "sizudra.cpp", "parts_latent.cpp", "parts_moe.cpp", "parts_stream.cpp", "parts_recurrent.cpp", "piditar.cpp", "parts_streams.cpp", "parts_linear_attention.cpp", "parts_pooled.cpp", "povipel.cpp", "plugin.cpp", "qwen2.cpp", "spec.cpp", "step.cpp", "store.cpp", "trace.cpp", "weights.cpp")]
 HOST_HEADERS = ["tq_engine.h"] + ["engine/" + n for n in (
     "config.h", "core.h", "engine.h", "generate.h", "json.h", "kernels.h", "linear.h", "model.h", "parts.h", "plugin.h", "spec.h",
     "step.h", "store.h", "trace.h", "weights.h")]

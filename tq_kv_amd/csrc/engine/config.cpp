@@ -15,7 +15,7 @@ std::vector<Architecture>& architectures() {
     return a;
 }
 std::once_flag g_builtin_once;
-void ensure_builtin() { std::call_once(g_builtin_once, [] { register_qwen2(); register_nikasun(); register_sizudra(); register_piditar(); }); }
+void ensure_builtin() { std::call_once(g_builtin_once, [] { register_qwen2(); register_nikasun(); register_sizudra(); register_piditar(); register_povipel(); }); }
 std::string joined(const std::vector<std::string>& v) {
     std::string s;
     for (size_t i = 0; i < v.size(); ++i) s += (i ? ", " : "") + v[i];

@@ -31,5 +31,6 @@ void register_qwen2();
 void register_nikasun();
 void register_sizudra();
 void register_piditar();
+void register_povipel();
 
 }  // namespace tq

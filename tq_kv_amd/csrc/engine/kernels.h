@@ -73,6 +73,7 @@ TQ_KERNEL(head_product, cptr, int, long long, long long, cptr, void*, int, long 
 TQ_KERNEL(moe_route, cptr, int, cptr, int, int, int, int, float, int, int32_t*, float*, cptr, float*, int, void*);
 TQ_KERNEL(moe_group, ci32, int, int, int, int, int32_t*, int32_t*, int32_t*, int32_t*, int32_t*, int32_t*, void*);
 TQ_KERNEL(moe_product, cptr, int, ci32, cptr, int, long long, void*, int, int, int, int, float, float, ci32, ci32, ci32, ci32, int, void*);
+TQ_KERNEL(moe_scale_rows, cptr, int, ci32, cf32, int, void*, float*, int, int, void*);
 TQ_KERNEL(moe_combine, cptr, int, ci32, cf32, int, cptr, cf32, void*, int, int, void*);
 TQ_KERNEL(pair_embed, cptr, int, int, long long, long long, ci32, ci32, ci32, ci32, ci32, int32_t*, float*, int, int, int, void*, int, void*);
 TQ_KERNEL(remember_tokens, ci32, ci32, ci32, ci32, int32_t*, int, void*);
@@ -105,6 +106,24 @@ TQ_KERNEL(attention_masked_mfma, cptr, cptr, cptr, ci32, ci32, int, int, int, in
           void*, int, int, int, int, void*);
 TQ_KERNEL(attention_masked, cptr, cptr, cptr, int, ci32, ci32, ci32, int, int, int, int, int, float, float, cptr, int, void*, int, int, int, int,
           int, void*);
+TQ_QUERY(int, streams_max);
+TQ_KERNEL(streams_fill, cf32, float*, int, int, int, void*);
+TQ_KERNEL(streams_step, float*, int, cptr, int, cf32, cf32, cf32, cf32, cf32, float, float*, void*, int, int, int, void*);
+TQ_KERNEL(add_layer_norm, float*, cptr, int, ci32, int, cf32, cf32, float, void*, int, int, int, void*);
+TQ_KERNEL(token_shift, cf32, cf32, float*, long long, ci32, ci32, ci32, ci32, void*, int, int, int, int, void*);
+TQ_KERNEL(shift_remember, cf32, float*, long long, ci32, ci32, ci32, int, int, void*);
+TQ_QUERY(int, linear_attention_max_dim);
+TQ_KERNEL(linear_attention, cptr, cptr, cptr, int, long long, cf32, long long, cf32, float, cf32, float, float, cf32, cf32, int, int, int, ci32, float*,
+          long long, ci32, ci32, ci32, ci32, ci32, float*, float*, float*, int, int, int, int, int, void*);
+TQ_KERNEL(head_norm_gate, cf32, cf32, float, cptr, int, long long, void*, int, int, int, int, void*);
+TQ_QUERY(int, pooled_attention_max_dim);
+TQ_QUERY(int, pooled_rows, int);
+TQ_KERNEL(pooled_store, cptr, int, cf32, cf32, int, float, cf32, cf32, int, int, cf32, cf32, int, ci32, ci32, ci32, int, void*, void*, void*, int, int, int,
+          int, int, int, void*);
+TQ_KERNEL(pool_blocks, void*, void*, int, ci32, ci32, ci32, int, int, int, int, int, int, int, void*);
+TQ_KERNEL(pooled_attention, cptr, cptr, cptr, int, ci32, ci32, ci32, int, int, int, float, cf32, cf32, cf32, int, int, void*, int, int, int, int, int,
+          void*);
+TQ_KERNEL(normed_pair_sum, cptr, cptr, int, cf32, cf32, float, float, void*, int, int, int, void*);
 TQ_QUERY(int, argmax_scratch_floats, int, int);
 TQ_KERNEL(argmax, cf32, int, int, int32_t*, float*, void*);
 TQ_KERNEL(repeat_penalty, float*, int, int, ci32, ci32, ci32, int, ci32, int, float, void*);

@@ -101,6 +101,12 @@ struct Stream {
     int n_ss = 0;
     Norm* next_norm = nullptr;
     bool of_last_rows = false;
+    // The stream in several copies [tokens, copies, hidden] float32 (memory of the step), for blocks that keep more than one; then
+    // `pending` is an update of all copies, X'[r] = sum_s copies_mix[s, r] X[s] + copies_out[r] pending, and h is not kept up to date
+    // until the last block writes the copies' sum there.
+    Tensor copies;
+    const float* copies_mix = nullptr;
+    const float* copies_out = nullptr;
     Tensor copy;                        // h in the activation type, where a kernel that added to h also wrote it (valid while copy_valid)
     bool copy_valid = false;
     void invalidate() { xw_for = nullptr; copy_valid = false; }
@@ -181,6 +187,7 @@ struct CacheEntry {
     int group = -1;                 // pages: which group's page table the step carries for it
     Tensor keys, values;            // pages: [pages, key_page...], [pages, value_page...]
     Tensor state;                   // state: [slots, shape...]; row `slot` is a sequence's
+    int64_t state_offset = 0;       // where in a slot's row the part's own state begins (a part that shares the row with others)
     bool writes = true;             // false: reads another run's cache
     int window = 0;
     int keep_first = 0;
@@ -231,5 +238,8 @@ void register_latent_parts();           // parts_latent.cpp; called by register_
 void register_moe_parts();              // parts_moe.cpp; likewise
 void register_stream_parts();           // parts_stream.cpp; likewise
 void register_recurrent_parts();        // parts_recurrent.cpp; likewise
+void register_streams_parts();          // parts_streams.cpp; likewise
+void register_linear_attention_parts(); // parts_linear_attention.cpp; likewise
+void register_pooled_parts();           // parts_pooled.cpp; likewise
 
 }  // namespace tq

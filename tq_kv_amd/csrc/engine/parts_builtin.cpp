@@ -947,6 +947,9 @@ void register_builtin_parts() {
         register_moe_parts();
         register_stream_parts();
         register_recurrent_parts();
+        register_streams_parts();
+        register_linear_attention_parts();
+        register_pooled_parts();
         register_kind("block", "pre_norm", [](const PartSpec& s, BuildEnv& e) { return std::make_shared<PreNormBlock>(s, e); });
     });
 }

@@ -14,9 +14,11 @@
 // Variants, all parameters: gated false makes an expert down(f(up_proj x)), f the gate's function of one product
 // (relu2: max(z, 0)^2), without a gate product and its tensor; normalize "chosen" makes the weights the softmax over
 // the chosen logits alone (times router_scale); shared_gate names a tensor [1, hidden] whose product with x, through
-// a sigmoid, multiplies the shared expert's output token by token.
+// a sigmoid, multiplies the shared expert's output token by token; score "sigmoid" makes an expert's score sigmoid(z) on its own
+// instead of the softmax over all; weight_on "input" multiplies an expert's input by the weight (the output is then the plain sum of
+// E(w x) over the chosen experts, which is not w E(x) since an expert is not linear).
 //
-// params: hidden, inter, n_experts, top, router_scale, gate / limit / alpha, gated, normalize, shared (a feed-forward
+// params: hidden, inter, n_experts, top, router_scale, gate / limit / alpha, gated, normalize, score, weight_on, shared (a feed-forward
 // part spec, or null), shared_gate (a tensor's name, or null); optional names {router, expert (with %d for the expert's number), gate, up,
 // down, shared}.  Tensors: router [experts, hidden]; per expert gate, up [inter, hidden], down
 // [hidden, inter]; the shared expert's own under its prefix.
@@ -48,6 +50,12 @@ public:
         const std::string normalize = r.string_or("normalize", "all");
         if (normalize != "all" && normalize != "chosen") raise(TQE_ERR_ARGUMENT, "routed_experts: unknown normalize '%s' (known: all, chosen)", normalize.c_str());
         renormalize_ = normalize == "chosen";
+        const std::string score = r.string_or("score", "softmax");
+        if (score != "softmax" && score != "sigmoid") raise(TQE_ERR_ARGUMENT, "routed_experts: unknown score '%s' (known: sigmoid, softmax)", score.c_str());
+        sigmoid_scores_ = score == "sigmoid";
+        const std::string weight_on = r.string_or("weight_on", "output");
+        if (weight_on != "output" && weight_on != "input") raise(TQE_ERR_ARGUMENT, "routed_experts: unknown weight_on '%s' (known: input, output)", weight_on.c_str());
+        weight_on_input_ = weight_on == "input";
         n_shared_gate_ = r.string_or("shared_gate", "");
         if (top_ > n_experts_) raise(TQE_ERR_ARGUMENT, "routed_experts: top %d of %d experts", top_, n_experts_);
         const int most = K::moe_max_experts.raw();
@@ -143,7 +151,7 @@ public:
         Tensor shared_scale;
         const bool gate_in_route = shared_gate_ && shared_gate_->t.dtype == router_->t.dtype;
         if (shared_gate_) shared_scale = c.alloc(F32, {n});
-        K::moe_route(x.x.data, dtype, router_->t.data, router_->t.dtype, n_experts_, (int)hidden_, top_, router_scale_, renormalize_ ? 1 : 0, (int32_t*)idx.data,
+        K::moe_route(x.x.data, dtype, router_->t.data, router_->t.dtype, n_experts_, (int)hidden_, top_, router_scale_, (renormalize_ ? 1 : 0) | (sigmoid_scores_ ? 2 : 0), (int32_t*)idx.data,
                      (float*)weight.data, gate_in_route ? shared_gate_->t.data : nullptr, gate_in_route ? (float*)shared_scale.data : nullptr, (int)n, c.stream);
         K::moe_group((const int32_t*)idx.data, (int)n, top_, n_experts_, tile_m, (int32_t*)pair_pos.data, (int32_t*)sorted_tok.data, tile_expert, tile_row0,
                      tile_rows, (int32_t*)n_tiles.data, c.stream);
@@ -157,21 +165,33 @@ public:
         const long long first_stride = (long long)(gated_ ? 2 : 1) * inter_ * hidden_;
         Tensor act = c.alloc(dtype, {pairs, inter_});
         Tensor y = c.alloc(dtype, {pairs, hidden_});
+        // the weight on the experts' inputs: every pair's row is its token's times the pair's weight, and the sum below is a plain one
+        const void* first_in = x.x.data;
+        const int32_t* first_rows = (const int32_t*)sorted_tok.data;
+        const float* sum_weight = (const float*)weight.data;
+        if (weight_on_input_) {
+            Tensor scaled = c.alloc(dtype, {pairs, hidden_}), unit = c.alloc(F32, {n, top_});
+            K::moe_scale_rows(x.x.data, dtype, (const int32_t*)pair_pos.data, (const float*)weight.data, top_, scaled.data, (float*)unit.data, (int)n, (int)hidden_,
+                              c.stream);
+            first_in = scaled.data;
+            first_rows = nullptr;
+            sum_weight = (const float*)unit.data;
+        }
         if (on_cores) {
-            K::moe_product_mfma(x.x.data, (const int32_t*)sorted_tok.data, gate_up_->t.data, first_stride, act.data, (int)inter_,
+            K::moe_product_mfma(first_in, first_rows, gate_up_->t.data, first_stride, act.data, (int)inter_,
                                 (int)hidden_, first, gate_.kind, gate_.limit, gate_.alpha, tile_expert, tile_row0, tile_rows,
                                 (const int32_t*)n_tiles.data, max_tiles, tile_m, c.stream);
             K::moe_product_mfma(act.data, nullptr, down_->t.data, (long long)(hidden_ * inter_), y.data, (int)hidden_, (int)inter_, 0, 0, 0.f, 1.f,
                                 tile_expert, tile_row0, tile_rows, (const int32_t*)n_tiles.data, max_tiles, tile_m, c.stream);
         } else {
-            K::moe_product(x.x.data, dtype, (const int32_t*)sorted_tok.data, gate_up_->t.data, gate_up_->t.dtype, first_stride,
+            K::moe_product(first_in, dtype, first_rows, gate_up_->t.data, gate_up_->t.dtype, first_stride,
                            act.data, (int)inter_, (int)hidden_, first, gate_.kind, gate_.limit, gate_.alpha, tile_expert, tile_row0, tile_rows,
                            (const int32_t*)n_tiles.data, max_tiles, c.stream);
             K::moe_product(act.data, dtype, nullptr, down_->t.data, down_->t.dtype, (long long)(hidden_ * inter_), y.data, (int)hidden_, (int)inter_, 0,
                            0, 0.f, 1.f, tile_expert, tile_row0, tile_rows, (const int32_t*)n_tiles.data, max_tiles, c.stream);
         }
         Tensor out = c.alloc(dtype, {n, hidden_});
-        K::moe_combine(y.data, dtype, (const int32_t*)pair_pos.data, (const float*)weight.data, top_, shared_out.data,
+        K::moe_combine(y.data, dtype, (const int32_t*)pair_pos.data, sum_weight, top_, shared_out.data,
                        shared_gate_ ? (const float*)shared_scale.data : nullptr, out.data, (int)n,
                        (int)hidden_, c.stream);
         return out;
@@ -182,7 +202,7 @@ private:
     int n_experts_, top_;
     float router_scale_;
     Gate gate_;
-    bool gated_ = true, renormalize_ = false;
+    bool gated_ = true, renormalize_ = false, sigmoid_scores_ = false, weight_on_input_ = false;
     std::string n_shared_gate_;
     OwnedPtr shared_gate_;
     std::string n_router_, n_expert_, n_gate_, n_up_, n_down_, n_shared_;

@@ -156,7 +156,7 @@ public:
         const int64_t n = x.rows();
         const int dtype = x.lazy ? BF16 : x.x.dtype;
         const long long row = entry.state.cols(), conv_part = (long long)(taps_ - 1) * width_;
-        float* state = (float*)entry.state.data;
+        float* state = (float*)entry.state.data + entry.state_offset;
         const Tensor yx = x.lazy ? linear_of_norm(c, x.norm, w_yx_, dtype) : linear(c, x.x, w_yx_, nullptr, dtype).t;
         Tensor u = c.alloc(F32, {n, width_}), a = c.alloc(F32, {n, width_}), g = c.alloc(F32, {n, width_});
         if (c.all_decode) {
@@ -279,7 +279,7 @@ public:
         const int64_t n = x.rows();
         const int dtype = x.lazy ? BF16 : x.x.dtype;
         const long long row = entry.state.cols(), conv_part = (long long)(taps_ - 1) * conv_ch_;
-        float* state = (float*)entry.state.data;
+        float* state = (float*)entry.state.data + entry.state_offset;
         const Tensor zxbcdt = x.lazy ? linear_of_norm(c, x.norm, w_in_, dtype) : linear(c, x.x, w_in_, nullptr, dtype).t;          // [z | x | B | C | dt | padding]
         Tensor xbc = c.alloc(F32, {n, conv_ch_}), y = c.alloc(F32, {n, inner_});
         if (c.all_decode) {

@@ -26,6 +26,11 @@ Json TensorSpec::to_json() const {
     j.set("init", init);
     j.set("std", std_dev);
     j.set("dtype", dtype);
+    if (!free.empty()) {
+        Json f = Json::array();
+        for (int d : free) f.push(Json(d));
+        j.set("free", f);
+    }
     return j;
 }
 
@@ -35,6 +40,8 @@ TensorSpec TensorSpec::from_json(const Json& j) {
     if (j["init"].is_string()) t.init = j["init"].as_string();
     if (j["std"].is_number()) t.std_dev = j["std"].as_number();
     if (j["dtype"].is_string()) t.dtype = j["dtype"].as_string();
+    if (j["free"].is_array())
+        for (const Json& d : j["free"].items()) t.free.push_back((int)d.as_int());
     if (t.dtype != "float" && t.dtype != "int32") raise(TQE_ERR_ARGUMENT, "tensor spec: dtype must be \"float\" or \"int32\", got \"%s\"", t.dtype.c_str());
     return t;
 }
@@ -64,6 +71,10 @@ Json CacheNeed::to_json() const {
         j.set("value_page", shape_json(value_page));
         j.set("window", window > 0 ? Json(window) : Json());
         if (keep_first > 0) j.set("keep_first", keep_first);
+        if (has_state()) {
+            j.set("state_shape", shape_json(state_shape));
+            j.set("state_dtype", dtype_name(state_dtype));
+        }
     } else {
         j.set("kind", "state");
         j.set("shape", shape_json(state_shape));
@@ -84,6 +95,14 @@ CacheNeed CacheNeed::from_json(const Json& j) {
         if (n.window < 0) raise(TQE_ERR_ARGUMENT, "cache need: window %d", n.window);
         if (j["keep_first"].is_int()) n.keep_first = (int)j["keep_first"].as_int();
         if (n.keep_first < 0) raise(TQE_ERR_ARGUMENT, "cache need: keep_first %d", n.keep_first);
+        if (!j["state_shape"].is_null()) {
+            n.state_shape = shape_from(j["state_shape"], "cache need");
+            const std::string dt = j["state_dtype"].is_string() ? j["state_dtype"].as_string() : "float32";
+            if (dt == "float32") n.state_dtype = F32;
+            else if (dt == "bfloat16") n.state_dtype = BF16;
+            else if (dt == "int32") n.state_dtype = I32;
+            else raise(TQE_ERR_ARGUMENT, "state of kind '%s' (known: bfloat16, float32, int32)", dt.c_str());
+        }
     } else if (kind == "state") {
         n.kind = State;
         n.state_shape = shape_from(j["shape"], "cache need");

@@ -16,8 +16,11 @@ namespace tq {
 // One named tensor of a part.  init: how the random-weights mode fills it: "normal" (N(0, std)),
 // "one_plus_normal" (1 + N(0, std)), "zeros", or a kind registered with register_init.
 // dtype: "float" follows the run's weight dtype; "int32" is an integer table.
+// free: dimensions whose size the checkpoint decides (a rank that no configuration key names); the size given here is what random
+// weights get, and the part reads the loaded tensor's own.
 struct TensorSpec {
     std::vector<int64_t> shape;
+    std::vector<int> free;
     std::string init = "normal";
     double std_dev = 0.02;
     std::string dtype = "float";
@@ -42,7 +45,8 @@ struct PartSpec {
 // What a mixer keeps per sequence.  Pages: keys and values for every position, in pages of
 // TQE_PAGE positions whose layout is the mixer's own: key_page and value_page are the shapes
 // of one page (window > 0: only the last `window` positions are ever read, and the first `keep_first`).  State: a
-// fixed-size row per sequence, zero at the start.
+// fixed-size row per sequence, zero at the start.  A need of pages may name a state_shape too (a block whose mixer keeps
+// keys and values and a fixed-size state beside them): such a run gets both.
 struct CacheNeed {
     enum Kind { None = 0, Pages = 1, State = 2 };
     int kind = None;
@@ -51,6 +55,9 @@ struct CacheNeed {
     int keep_first = 0;          // with a window: the sequence's first positions that stay visible whatever the window
     std::vector<int64_t> state_shape;
     int state_dtype = F32;
+    bool has_state() const { return !state_shape.empty(); }
+    bool same_pages(const CacheNeed& o) const { return key_page == o.key_page && value_page == o.value_page && window == o.window && keep_first == o.keep_first; }
+    bool same_state(const CacheNeed& o) const { return state_shape == o.state_shape && state_dtype == o.state_dtype; }
     bool operator==(const CacheNeed& o) const {
         return kind == o.kind && key_page == o.key_page && value_page == o.value_page && window == o.window && keep_first == o.keep_first &&
                state_shape == o.state_shape && state_dtype == o.state_dtype;

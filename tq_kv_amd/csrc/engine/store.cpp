@@ -17,24 +17,28 @@ CacheStore::CacheStore(const std::vector<CacheNeed>& needs, const std::vector<in
     n_pages = holds_pages ? (int)(max_tokens / TQE_PAGE) : 0;
     max_slots = holds_pages ? std::max(1, std::min(max_slots_, n_pages)) : std::max(1, max_slots_);
 
-    struct Place { bool pages; size_t group; int index; };
-    std::vector<Place> place(n_runs, Place{false, 0, -1});
+    // where a run's pages and its state row lie (a run may have both)
+    struct Place { int page_group = -1, page_index = -1, state_group = -1, state_index = -1; };
+    std::vector<Place> place(n_runs);
     for (size_t r = 0; r < n_runs; ++r) {
         const CacheNeed& need = needs[r];
         if (need.kind == CacheNeed::None || cache_of[r] >= 0) continue;
         if (need.kind == CacheNeed::Pages) {
             size_t g = 0;
             for (; g < page_groups.size(); ++g)
-                if (page_groups[g].need == need) break;
+                if (page_groups[g].need.same_pages(need)) break;
             if (g == page_groups.size()) { page_groups.emplace_back(); page_groups[g].need = need; page_groups[g].n_pages = n_pages; }
-            place[r] = Place{true, g, (int)page_groups[g].runs.size()};
+            place[r].page_group = (int)g;
+            place[r].page_index = (int)page_groups[g].runs.size();
             page_groups[g].runs.push_back((int)r);
-        } else {
+        }
+        if (need.kind == CacheNeed::State || need.has_state()) {
             size_t g = 0;
             for (; g < state_groups.size(); ++g)
-                if (state_groups[g].need == need) break;
+                if (state_groups[g].need.same_state(need)) break;
             if (g == state_groups.size()) { state_groups.emplace_back(); state_groups[g].need = need; }
-            place[r] = Place{false, g, (int)state_groups[g].runs.size()};
+            place[r].state_group = (int)g;
+            place[r].state_index = (int)state_groups[g].runs.size();
             state_groups[g].runs.push_back((int)r);
         }
     }
@@ -71,7 +75,7 @@ CacheStore::CacheStore(const std::vector<CacheNeed>& needs, const std::vector<in
         if (need.kind == CacheNeed::None) continue;
         const int src = cache_of[r];
         const size_t owner = src < 0 ? r : (size_t)src;
-        if (owner >= n_runs || place[owner].index < 0) {
+        if (owner >= n_runs || (place[owner].page_index < 0 && place[owner].state_index < 0)) {
             tqe_cache_free(book);
             book = nullptr;
             raise(TQE_ERR_ARGUMENT, "run %zu reads the cache of run %zu, which keeps none", r, owner);
@@ -85,21 +89,22 @@ CacheStore::CacheStore(const std::vector<CacheNeed>& needs, const std::vector<in
         e.kind = need.kind;
         e.writes = src < 0;
         const Place& p = place[owner];
-        if (p.pages) {
-            const PageGroup& g = page_groups[p.group];
-            e.group = (int)p.group;
+        if (p.page_index >= 0) {
+            const PageGroup& g = page_groups[(size_t)p.page_group];
+            e.group = p.page_group;
             e.window = need.window;
             e.keep_first = need.keep_first;
-            e.keys = g.keys->t.slice(p.index, p.index + 1);
-            e.values = g.values->t.slice(p.index, p.index + 1);
+            e.keys = g.keys->t.slice(p.page_index, p.page_index + 1);
+            e.values = g.values->t.slice(p.page_index, p.page_index + 1);
             // drop the leading dimension of one run
             for (Tensor* t : {&e.keys, &e.values}) {
                 for (int i = 0; i + 1 < t->ndim; ++i) t->shape[i] = t->shape[i + 1];
                 --t->ndim;
             }
-        } else {
-            const StateGroup& g = state_groups[p.group];
-            e.state = g.state->t.slice(p.index, p.index + 1);
+        }
+        if (p.state_index >= 0) {
+            const StateGroup& g = state_groups[(size_t)p.state_group];
+            e.state = g.state->t.slice(p.state_index, p.state_index + 1);
             for (int i = 0; i + 1 < e.state.ndim; ++i) e.state.shape[i] = e.state.shape[i + 1];
             --e.state.ndim;
         }

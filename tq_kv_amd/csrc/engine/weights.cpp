@@ -205,7 +205,12 @@ void check_weights(const std::map<std::string, StoredTensor>& stored, const Tens
         const StoredTensor& st = it->second;
         // a scalar (no dimensions) and a tensor of one element are the same thing: that is how a scalar is held
         auto held_as = [](const std::vector<int64_t>& s) { return s.empty() ? std::vector<int64_t>{1} : s; };
-        if (held_as(st.shape) != held_as(w.second.shape)) {
+        // (a dimension the specification leaves to the checkpoint fits whatever its size)
+        std::vector<int64_t> expected = held_as(w.second.shape);
+        if (expected.size() == held_as(st.shape).size())
+            for (int d : w.second.free)
+                if (d >= 0 && (size_t)d < expected.size() && held_as(st.shape)[(size_t)d] > 0) expected[(size_t)d] = held_as(st.shape)[(size_t)d];
+        if (held_as(st.shape) != expected) {
             shape_lines.push_back("  Wrong shape: " + w.first + " is " + shape_text(st.shape) + ", expected " + shape_text(w.second.shape));
             Json e = Json::array();
             e.push(w.first);

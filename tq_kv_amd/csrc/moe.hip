@@ -2,7 +2,9 @@
 // expert, the experts' products over the grouped rows, and the weighted sum.
 //
 //   route     z = W_r x in float32, s = softmax(z) over all experts, the `top` largest (the lower index wins
-//             a tie); weight = s * scale, not renormalised.  One wave per token.
+//             a tie); weight = s * scale, not renormalised.  One wave per token.  Mode bit 1 renormalises over the chosen;
+//             mode bit 2 makes every expert's score sigmoid(z) on its own instead of the softmax.
+//   scale     rows[pair_pos[p]] = weight[p] * x[p / top] (for experts whose input, not output, carries the weight), and unit[p] = 1
 //   group     pair p = (token p / top, choice p % top) gets a row of its own among its expert's rows:
 //             pair_pos[p]; sorted_tok[row] names the row's token.  The rows of an expert are cut into tiles of
 //             tile_m rows; the tile list (expert, first row, rows) and its length stay on the device, so the
@@ -26,8 +28,9 @@
 // under way at once, added up in a fixed order), then the first wave takes the softmax and the largest.
 template <typename TA, typename TW>
 __global__ __launch_bounds__(MOE_ROUTE_WAVES * TQK_WAVE)
-void moe_route_kernel(const TA* __restrict__ x, const TW* __restrict__ w, int n_experts, int hidden, int top, float scale, int renormalize,
+void moe_route_kernel(const TA* __restrict__ x, const TW* __restrict__ w, int n_experts, int hidden, int top, float scale, int mode,
                       int32_t* __restrict__ idx, float* __restrict__ weight, const TW* __restrict__ gate_w, float* __restrict__ gate_out) {
+    const int renormalize = mode & 1, sigmoid_scores = mode & 2;
     __shared__ float z[MOE_MAX_EXPERTS];
     const int wave = threadIdx.x / TQK_WAVE, lane = threadIdx.x % TQK_WAVE;
     const int t = blockIdx.x;
@@ -92,7 +95,7 @@ void moe_route_kernel(const TA* __restrict__ x, const TW* __restrict__ w, int n_
         if (lane == best_e % TQK_WAVE) z[best_e] = -INFINITY;       // the lane that reads this expert writes it: no other sees it
         if (lane == 0) {
             idx[(size_t)t * top + k] = best_e;
-            weight[(size_t)t * top + k] = expf(best - m) / sum * scale;
+            weight[(size_t)t * top + k] = (sigmoid_scores ? 1.f / (1.f + expf(-best)) : expf(best - m) / sum) * scale;
         }
     }
     if (!renormalize) return;
@@ -240,13 +243,39 @@ void moe_combine_kernel(const TA* __restrict__ y, const int32_t* __restrict__ pa
     }
 }
 
+// ---- scale -----------------------------------------------------------------------------------
+template <typename TA>
+__global__ __launch_bounds__(256)
+void moe_scale_rows_kernel(const TA* __restrict__ x, const int32_t* __restrict__ pair_pos, const float* __restrict__ weight, int top,
+                           TA* __restrict__ rows, float* __restrict__ unit, int hidden) {
+    const size_t p = blockIdx.x;
+    const float w = weight[p];
+    const TA* src = x + (p / top) * hidden;
+    TA* dst = rows + (size_t)pair_pos[p] * hidden;
+    for (int i = threadIdx.x; i < hidden; i += blockDim.x) dst[i] = from_float<TA>(w * to_float(src[i]));
+    if (threadIdx.x == 0) unit[p] = 1.f;
+}
+
 // ---- entry points ----------------------------------------------------------------------------
+extern "C" int tqk_moe_scale_rows(const void* x, int act_dtype, const int32_t* pair_pos, const float* weight, int top, void* rows, float* unit,
+                                  int n_tokens, int hidden, void* stream) {
+    TQK_REQUIRE(x && pair_pos && weight && rows && unit, "tqk_moe_scale_rows: null pointer");
+    TQK_REQUIRE(top > 0 && hidden > 0 && n_tokens >= 0 && (long long)n_tokens * top <= 0x7fffffff, "tqk_moe_scale_rows: bad sizes");
+    if (n_tokens == 0) return 0;
+    hipStream_t s = (hipStream_t)stream;
+    const unsigned pairs = (unsigned)(n_tokens * top);
+    if (act_dtype == TQK_F32) moe_scale_rows_kernel<float><<<pairs, 256, 0, s>>>((const float*)x, pair_pos, weight, top, (float*)rows, unit, hidden);
+    else if (act_dtype == TQK_BF16) moe_scale_rows_kernel<bf16_t><<<pairs, 256, 0, s>>>((const bf16_t*)x, pair_pos, weight, top, (bf16_t*)rows, unit, hidden);
+    else return tqk_fail("tqk_moe_scale_rows: unknown dtype %d", act_dtype);
+    return tqk_check_launch("tqk_moe_scale_rows");
+}
+
 extern "C" int tqk_moe_max_experts(void) { return MOE_MAX_EXPERTS; }
 extern "C" int tqk_moe_tile_rows(void) { return MOE_TM; }
 extern "C" int tqk_moe_max_tiles(int n_pairs, int n_experts, int tile_m) { return (n_pairs + tile_m - 1) / tile_m + n_experts; }
 
 extern "C" int tqk_moe_route(const void* x, int act_dtype, const void* w_router, int w_dtype, int n_experts, int hidden, int top, float scale,
-                             int renormalize, int32_t* idx, float* weight, const void* gate_w, float* gate_out, int n_tokens, void* stream) {
+                             int mode, int32_t* idx, float* weight, const void* gate_w, float* gate_out, int n_tokens, void* stream) {
     TQK_REQUIRE(x && w_router && idx && weight, "tqk_moe_route: null pointer");
     TQK_REQUIRE(n_experts > 0 && n_experts <= MOE_MAX_EXPERTS, "tqk_moe_route: %d experts, the kernel takes 1 to %d", n_experts, MOE_MAX_EXPERTS);
     TQK_REQUIRE(top > 0 && top <= n_experts && hidden > 0 && n_tokens >= 0, "tqk_moe_route: bad sizes (top %d of %d experts)", top, n_experts);
@@ -254,7 +283,7 @@ extern "C" int tqk_moe_route(const void* x, int act_dtype, const void* w_router,
     if (n_tokens == 0) return 0;
     hipStream_t s = (hipStream_t)stream;
 #define TQK_ROUTE(TA, TW) \
-    moe_route_kernel<TA, TW><<<n_tokens, MOE_ROUTE_WAVES * TQK_WAVE, 0, s>>>((const TA*)x, (const TW*)w_router, n_experts, hidden, top, scale, renormalize, idx, weight, (const TW*)gate_w, gate_out)
+    moe_route_kernel<TA, TW><<<n_tokens, MOE_ROUTE_WAVES * TQK_WAVE, 0, s>>>((const TA*)x, (const TW*)w_router, n_experts, hidden, top, scale, mode, idx, weight, (const TW*)gate_w, gate_out)
     if (act_dtype == TQK_F32 && w_dtype == TQK_F32) TQK_ROUTE(float, float);
     else if (act_dtype == TQK_F32 && w_dtype == TQK_BF16) TQK_ROUTE(float, bf16_t);
     else if (act_dtype == TQK_BF16 && w_dtype == TQK_F32) TQK_ROUTE(bf16_t, float);

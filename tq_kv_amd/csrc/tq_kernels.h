@@ -245,12 +245,16 @@ int tqk_latent_values(const float* o, const void* w_uv, int w_dtype, const float
  * relu2 gives max(z, 0)^2).  tqk_moe_route with renormalize: the chosen weights are divided by their sum (the softmax over
  * the chosen logits alone); with gate_w [hidden] (of the router's type, or null) it also writes gate_out[t] = sigmoid(x[t] . gate_w).
  * tqk_moe_combine: out[t] = sum_k weight[t, k] y[pair_pos[t, k]] + shared_scale[t] * shared[t]
- * (shared may be null; shared_scale null: 1). */
+ * (shared may be null; shared_scale null: 1).  tqk_moe_route's mode: bit 1 is that renormalising, bit 2 makes the scores
+ * sigmoid(z) of every expert on its own instead of the softmax.  tqk_moe_scale_rows: rows[pair_pos[p]] = weight[p] * x[p / top]
+ * and unit[p] = 1, for experts whose input carries the weight. */
+int tqk_moe_scale_rows(const void* x, int act_dtype, const int32_t* pair_pos, const float* weight, int top, void* rows, float* unit,
+                       int n_tokens, int hidden, void* stream);
 int tqk_moe_max_experts(void);
 int tqk_moe_tile_rows(void);
 int tqk_moe_max_tiles(int n_pairs, int n_experts, int tile_m);
 int tqk_moe_route(const void* x, int act_dtype, const void* w_router, int w_dtype, int n_experts, int hidden, int top, float scale,
-                  int renormalize, int32_t* idx, float* weight, const void* gate_w, float* gate_out, int n_tokens, void* stream);
+                  int mode, int32_t* idx, float* weight, const void* gate_w, float* gate_out, int n_tokens, void* stream);
 int tqk_moe_group(const int32_t* idx, int n_tokens, int top, int n_experts, int tile_m, int32_t* pair_pos, int32_t* sorted_tok,
                   int32_t* tile_expert, int32_t* tile_row0, int32_t* tile_rows, int32_t* n_tiles, void* stream);
 int tqk_moe_product(const void* x, int act_dtype, const int32_t* x_rows, const void* w, int w_dtype, long long expert_stride, void* y,
@@ -415,6 +419,67 @@ int tqk_append_history(const int32_t* tokens, const int32_t* row_req, int32_t* h
 size_t tqk_sample_scratch_bytes(int n_rows, int vocab, int top_k, float top_p);
 int tqk_sample(const float* logits, int n_rows, int vocab, float temperature, int top_k, float top_p,
                const float* uniforms, int32_t* out, void* scratch, void* stream);
+
+/* The residual stream in several copies, a layer norm with weight and bias, the previous token mixed into a mixer's input (streams.hip).
+ * X [tokens, copies, width] float32.  tqk_streams_step: where y is given, X'[t, r] = sum_s mix[s, r] X[t, s] + out_w[r] y[t]; then, where
+ * in_w is given, u = sum_s in_w[s] X'[t, s] goes to u_out (if given) and (u - mean) / sqrt(var + eps) norm_w + norm_b to n_out (if given).
+ * tqk_add_layer_norm: out[i] = that norm of h[rows[i]] + delta[rows[i]] (rows null: row i; h or delta may be null; write_back leaves
+ * the sum in h).  tqk_token_shift: out[t] = n[t] + (n[t - 1] - n[t]) mu, with the sequence's state row in place of n[t - 1] for the first
+ * token a step brings of it; remember != 0 (steps of one token a sequence) also leaves n[t] in the state.  tqk_shift_remember: the state
+ * of every sequence becomes n of the last token the step brings of it. */
+int tqk_streams_max(void);
+int tqk_streams_fill(const float* h, float* X, int n_streams, int n_tokens, int width, void* stream);
+int tqk_streams_step(float* X, int n_streams, const void* y, int y_dtype, const float* mix, const float* out_w, const float* in_w,
+                     const float* norm_w, const float* norm_b, float eps, float* u_out, void* n_out, int n_dtype, int n_tokens, int width,
+                     void* stream);
+int tqk_add_layer_norm(float* h, const void* delta, int delta_dtype, const int32_t* rows, int n_rows, const float* weight, const float* bias,
+                       float eps, void* out, int out_dtype, int width, int write_back, void* stream);
+int tqk_token_shift(const float* n, const float* mu, float* state, long long state_stride, const int32_t* tok_seq, const int32_t* tok_pos,
+                    const int32_t* seq_start, const int32_t* seq_slot, void* out, int out_dtype, int n_tokens, int width, int remember,
+                    void* stream);
+int tqk_shift_remember(const float* n, float* state, long long state_stride, const int32_t* cu, const int32_t* seq_new, const int32_t* seq_slot,
+                       int n_seqs, int width, void* stream);
+
+/* Linear attention with a decaying state (linear_attention.hip): per head S_t = diag(a_t) S_(t-1) + k_t v_t^T, o_t = S_t^T q_t, the state
+ * of a slot [heads][d][dv] float32.  q, k, v: rows `stride` elements apart, heads side by side.  The decay: z [tokens, heads * d] float32
+ * with z_bias gives a = sigmoid(z + bias)^inv_tau per key channel; z null: head_decay[h] for the whole head.  q and k are turned by
+ * tok_pos through cos, sin [max_pos, rot_dim / 2] (style 1: halves, 2: pairs; cos null: not turned) and multiplied by q_scale, k_scale.
+ * mode 0: every sequence's tokens in order from its state row, which is written back (cu, seq_new, seq_slot; n_items sequences).
+ * mode 1 and 2: chunks as tqk_ssm_chunks takes them (chunk_row0, chunk_count; n_items chunks), between them tqk_chunk_carry with
+ * p_stride heads * d, p_div dv and per_seq heads * d * dv.  out [tokens, heads, dv] float32.
+ * tqk_head_norm_gate: out[t, h] = o[t, h] / rms(o[t, h]) * weight (null: 1) * silu(gate[t, h]) (null: 1). */
+int tqk_linear_attention_max_dim(void);
+int tqk_linear_attention(const void* q, const void* k, const void* v, int act_dtype, long long stride, const float* z, long long z_stride,
+                         const float* z_bias, float inv_tau, const float* head_decay, float q_scale, float k_scale, const float* cos,
+                         const float* sin, int rot_dim, int style, int max_pos, const int32_t* tok_pos, float* state, long long state_stride,
+                         const int32_t* cu, const int32_t* seq_new, const int32_t* seq_slot, const int32_t* chunk_row0,
+                         const int32_t* chunk_count, float* chunk_state, float* chunk_decay, float* out, int mode, int n_items, int heads,
+                         int d, int dv, void* stream);
+int tqk_head_norm_gate(const float* o, const float* weight, float eps, const void* gate, int gate_dtype, long long gate_stride, void* out,
+                       int out_dtype, int n_tokens, int heads, int dv, void* stream);
+
+/* Attention over a window plus pooled blocks (pooled_attention.hip).  Pages: keys [kv heads][page + tqk_pooled_rows(pool)][d], values
+ * likewise with dv; a block's means lie behind the positions of the page that holds its last position.  tqk_pooled_store: qkv
+ * [tokens, (heads + kv heads) d + kv heads dv]; normed: q and k heads are divided by their root mean square (times q_weight, k_weight
+ * [d] if given); then their first rot_dim elements are turned (style 0: not); vcos given: values are turned over all dv elements in
+ * the same layout.  tqk_pool_blocks: the means of the blocks that end among the step's positions.  tqk_pooled_attention: row r
+ * (sequence row_seq[r], position row_pos[r]) sees positions j with 0 <= pos - j < window and every block that ends at or before
+ * pos - window; sink [heads] float32 or null; vcos given: the output is turned back by the row's position. */
+int tqk_pooled_attention_max_dim(void);
+int tqk_pooled_rows(int pool);
+int tqk_pooled_store(const void* qkv, int dtype, const float* q_weight, const float* k_weight, int normed, float eps, const float* cos,
+                     const float* sin, int rot_dim, int style, const float* vcos, const float* vsin, int max_pos, const int32_t* tok_seq,
+                     const int32_t* tok_pos, const int32_t* table, int width, void* keys, void* values, void* q_out, int n_tokens,
+                     int heads, int kv_heads, int d, int dv, int pool, void* stream);
+int tqk_pool_blocks(void* keys, void* values, int dtype, const int32_t* seq_start, const int32_t* seq_new, const int32_t* table, int width,
+                    int n_seqs, int max_new, int pool, int kv_heads, int d, int dv, void* stream);
+int tqk_pooled_attention(const void* q, const void* keys, const void* values, int dtype, const int32_t* row_seq, const int32_t* row_pos,
+                         const int32_t* table, int width, int window, int pool, float scale, const float* sink, const float* vcos,
+                         const float* vsin, int style, int max_pos, void* out, int n_rows, int heads, int kv_heads, int d, int dv,
+                         void* stream);
+/* out[t] = c (x[t] / rms(x[t]) wx + y[t] / rms(y[t]) wy) over rows of `width` elements (streams.hip) */
+int tqk_normed_pair_sum(const void* x, const void* y, int dtype, const float* wx, const float* wy, float eps, float c, void* out, int out_dtype,
+                        int n_tokens, int width, void* stream);
 
 #ifdef __cplusplus
 }

@@ -12,7 +12,7 @@ import torch
 from ..csrc import build as _build
 
 _LIB = None
-KERNEL_ABI = 21         # tqk_abi_version of the kernel library these wrappers are written against
+KERNEL_ABI = 22         # tqk_abi_version of the kernel library these wrappers are written against
 
 F32, BF16 = 0, 1
 STYLE_NONE, STYLE_HALVES, STYLE_PAIRS = 0, 1, 2

@@ -78,6 +78,8 @@ class KVNeed:
     key_page: Optional[Tuple[int, ...]] = None
     value_page: Optional[Tuple[int, ...]] = None
     keep_first: int = 0         # with a window: the sequence's first positions that stay visible (their pages are kept)
+    state_shape: Optional[Tuple[int, ...]] = None       # a fixed-size state row beside the pages (a mixer that keeps both)
+    state_dtype: str = "float32"
 
     def pages(self):
         page = native.page_size()
@@ -90,6 +92,9 @@ class KVNeed:
         j = {"kind": "pages", "key_page": list(key), "value_page": list(value), "window": self.window}
         if self.keep_first:
             j["keep_first"] = int(self.keep_first)
+        if self.state_shape is not None:
+            j["state_shape"] = [int(v) for v in self.state_shape]
+            j["state_dtype"] = self.state_dtype
         return j
 
 
@@ -113,9 +118,10 @@ def need_from_json(j):
         return StateNeed(tuple(j["shape"]), j.get("dtype", "float32"))
     key, value = tuple(j["key_page"]), tuple(j["value_page"])
     page = native.page_size()
+    state = {"state_shape": tuple(j["state_shape"]), "state_dtype": j.get("state_dtype", "float32")} if j.get("state_shape") is not None else {}
     if len(key) == 3 and len(value) == 3 and key[1] == page and value[2] == page and key[0] == value[0]:
-        return KVNeed(key[0], key[2], j.get("window"), None if value[1] == key[2] else value[1], keep_first=j.get("keep_first", 0))
-    return KVNeed(window=j.get("window"), key_page=key, value_page=value, keep_first=j.get("keep_first", 0))
+        return KVNeed(key[0], key[2], j.get("window"), None if value[1] == key[2] else value[1], keep_first=j.get("keep_first", 0), **state)
+    return KVNeed(window=j.get("window"), key_page=key, value_page=value, keep_first=j.get("keep_first", 0), **state)
 
 
 def need_to_json(need):
