@@ -20,7 +20,8 @@ Nikasun design (attention through cached latents with a window, routed experts) 
 model's layers, beside a Qwen2 shape of the same width, depth, heads and active feed-forward size: prompt pass and
 decoding of both, tokens a second.  `python bench.py --masked` does the same for the Sizudra design (attention with normed
 heads, mixed values, and in every other layer a score cap, a window that keeps the first positions and a sink; a pair
-embedding; norms on the parts' outputs; routed experts without a gate product).  `python bench.py --recurrent` does it for the
+embedding; norms on the parts' outputs; routed experts without a gate product).  `python bench.py --streams` does it for the Povipel design beside a
+Piditar shape of equal size.  `python bench.py --recurrent` does it for the
 Piditar design (layers of attention, of a real-gated linear recurrent unit and of a selective state-space mixer, each with a dense
 feed-forward).
 """
@@ -52,6 +53,7 @@ def main():
     ap.add_argument("--latent-sizes", default="2048,4096", help="widths of the --latent and --masked comparisons")
     ap.add_argument("--masked", action="store_true", help="measure the Sizudra design beside a Qwen2 shape of equal size instead of the default workload")
     ap.add_argument("--recurrent", action="store_true", help="measure the Piditar design beside a Qwen2 shape of equal size instead of the default workload")
+    ap.add_argument("--streams", action="store_true", help="measure the Povipel design beside a Piditar shape of equal size instead of the default workload")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this library runs on one GPU; --gpus %d is not supported" % args.gpus)
@@ -162,6 +164,8 @@ def main():
 
     if args.recurrent:
         return design_comparison("piditar", recurrent_shapes, args, torch, Model, Engine, note, timed_prefill, decode, random_prompts, release)
+    if args.streams:
+        return design_comparison("povipel", streams_shapes, args, torch, Model, Engine, note, timed_prefill, decode, random_prompts, release, beside="piditar")
 
     # -- the headline shape -------------------------------------------------------------------------
     raw = dict(catalog.find(args.shape))
@@ -364,12 +368,36 @@ def recurrent_shapes(width, layers=4):
                             "mamba2_heads": mamba2["heads"], "mamba2_state": 128, "conv": 4}
 
 
-def design_comparison(design, shapes, args, torch, Model, Engine, note, timed_prefill, decode, random_prompts, release):
+def streams_shapes(width, layers=4):
+    """A Povipel configuration (the stream in four copies; attention over a window plus pooled blocks beside a gated linear attention, and
+    retention, in turn; a dense feed-forward and routed experts in turn) and a Piditar one (attention, recurrent unit, state-space mixer,
+    recurrent unit; gated dense feed-forwards) of the same width, depth, attention heads and head size, and as many multiply-adds in the
+    active feed-forward products."""
+    piditar, _, base = recurrent_shapes(width, layers)
+    heads, dim, kv_heads = base["heads"], 128, base["kv_heads"]
+    left = {"heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": dim, "scale": dim ** -0.5, "mask": {"size": 1024, "pool": 16}, "rot": {"base": 10000.0, "dims": 64}}
+    right = {"heads": width // 256, "dim": 128, "vdim": 256, "tau": 16.0}
+    retention = {"heads": width // 128, "dim": 128, "vdim": 256, "rot": {"base": 10000.0, "dims": 128},
+                 "decay": [1.0 - 2.0 ** (-5.0 - 3.0 * h / max(1, width // 128 - 1)) for h in range(width // 128)]}
+    # a gated feed-forward of 3 W holds 9 W^2 weights: the same in two products, and in the three products of each of 4 chosen experts
+    dense = {"kind": "dense", "ff": 9 * width // 2}
+    moe = {"kind": "moe", "expert": {"ff": 3 * width // 4}, "router": {"experts": 32, "top": 4}}
+    kinds = [("parallel", {"left": left, "right": right}, dense), ("retention", retention, moe), ("parallel", {"left": left, "right": right}, moe),
+             ("retention", retention, dense)]
+    lay = [{"type": kinds[l % 4][0], "mixer": kinds[l % 4][1], "mlp": kinds[l % 4][2]} for l in range(layers)]
+    povipel = {"architecture": "Povipel", "vocab": 32000, "width": width, "embedding": {"scale": width ** 0.5}, "norm": {"eps": 1e-5}, "streams": 4,
+               "logit_softcap": 30.0, "layers": lay, "loop": {"start": 0, "stop": layers, "times": 1}, "max_positions": 8192}
+    return povipel, piditar, {"width": width, "layers": layers, "heads": heads, "kv_heads": kv_heads, "streams": 4, "window": 1024, "pool": 16,
+                              "linear_heads": right["heads"], "linear_dim": 128, "linear_vdim": 256, "retention_heads": retention["heads"],
+                              "dense_ff": dense["ff"], "experts": 32, "top": 4, "expert_ff": moe["expert"]["ff"], "beside_ff": base["ff"]}
+
+
+def design_comparison(design, shapes, args, torch, Model, Engine, note, timed_prefill, decode, random_prompts, release, beside="qwen2"):
     prompt_len, out = 2048, {}
     for width in [int(x) for x in args.latent_sizes.split(",")]:
         other, qwen2, sizes = shapes(width)
         row = {"sizes": sizes}
-        for name, raw in ((design, other), ("qwen2", qwen2)):
+        for name, raw in ((design, other), (beside, qwen2)):
             note("width %d, %s: random weights" % (width, name))
             model = Model.random(raw, seed=0, dtype="bfloat16", device="cuda:0")
             engine = Engine(model, max_tokens=64 * (prompt_len + 256))
@@ -386,13 +414,13 @@ def design_comparison(design, shapes, args, torch, Model, Engine, note, timed_pr
             engine = model = None
             release()
         for key in ("prefill_tok_s", "decode_b8_tok_s", "decode_b64_tok_s"):
-            row["ratio_" + key] = round(row[design + "_" + key] / row["qwen2_" + key], 3)
+            row["ratio_" + key] = round(row[design + "_" + key] / row[beside + "_" + key], 3)
         out["width_%d" % width] = row
     first = out["width_%d" % int(args.latent_sizes.split(",")[0])]
     print(json.dumps({"metric": "decode tok/s @ batch 8, %s design at width %s" % (design.capitalize(), args.latent_sizes.split(",")[0]),
                       "value": first[design + "_decode_b8_tok_s"], "unit": "tokens/s", "n_gpus": 1, "steps": min(args.steps, 32), "warmup": 4,
                       "ms_per_step": first[design + "_decode_b8_ms"], "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
-                      "dtype": "bf16", "data": "synthetic", "config": {"model": design + " beside qwen2 at equal size", "prompt_len": prompt_len,
+                      "dtype": "bf16", "data": "synthetic", "config": {"model": design + " beside " + beside + " at equal size", "prompt_len": prompt_len,
                                                                      "weights": "random"}, "comparison": out}))
     return 0
 

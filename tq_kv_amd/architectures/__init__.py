@@ -1,3 +1,3 @@
 """Architectures: the Python mirrors of their typed configurations (the architectures themselves
 are registered in the engine library, one file each under csrc/engine/)."""
-from . import nikasun, piditar, qwen2, sizudra  # noqa: F401
+from . import nikasun, piditar, povipel, qwen2, sizudra  # noqa: F401

@@ -12,7 +12,8 @@
 //                      Its pages keep the blocks' means behind the positions: keys [kv heads][page + ceil(page / pool)][head_dim],
 //                      values likewise with value_dim; a block lies in the page of its last position.  The cache keeps every page.
 //                      params: hidden, n_heads, n_kv_heads, head_dim, value_dim, scale, window, pool, qk_norm, eps, sink,
-//                      rotate_values, position (a part spec with tables), value_position (a part spec: the values' tables), names
+//                      rotate_values, position (a part spec with tables, or null: q and k are not turned), value_position (a part spec:
+//                      the values' tables, whose layout is then the one that counts), names
 //                      {q, k, v, o, q_norm, k_norm, sink}.
 //   parallel           c (n_a(a(x)) + n_b(b(x))): two mixers read the same input, each output is divided by its root mean square over
 //                      the model's width and multiplied by a weight of its own, and the two are added and scaled (c = 1/2).  One of
@@ -80,12 +81,12 @@ public:
         auto name = [&](const char* role, const char* fallback) { return names[role].is_string() ? names[role].as_string() : std::string(fallback); };
         n_q_ = name("q", "q_proj.weight"); n_k_ = name("k", "k_proj.weight"); n_v_ = name("v", "v_proj.weight"); n_o_ = name("o", "o_proj.weight");
         n_q_norm_ = name("q_norm", "q_norm.weight"); n_k_norm_ = name("k_norm", "k_norm.weight"); n_sink_ = name("sink", "sink");
-        position_ = shared_position(spec.params["position"], "pooled_attention: position", env);
-        if (position_->tables().rot_dim > head_dim_) raise(TQE_ERR_ARGUMENT, "pooled_attention: %d turned elements in heads of %d", position_->tables().rot_dim, head_dim_);
+        if (!spec.params["position"].is_null()) position_ = shared_position(spec.params["position"], "pooled_attention: position", env);
+        if (position_ && position_->tables().rot_dim > head_dim_) raise(TQE_ERR_ARGUMENT, "pooled_attention: %d turned elements in heads of %d", position_->tables().rot_dim, head_dim_);
         if (rotate_values_) {
             value_position_ = shared_position(spec.params["value_position"], "pooled_attention: value_position", env);
-            const Position::Tables vt = value_position_->tables(), qt = position_->tables();
-            if (vt.rot_dim != value_dim_ || vt.style != qt.style || vt.style == STYLE_NONE)
+            const Position::Tables vt = value_position_->tables();
+            if (vt.rot_dim != value_dim_ || vt.style == STYLE_NONE || (position_ && position_->tables().style != STYLE_NONE && position_->tables().style != vt.style))
                 raise(TQE_ERR_ARGUMENT, "pooled_attention: values are turned over all their %d elements, in the layout of the keys", value_dim_);
         }
         graph_safe = true;
@@ -139,23 +140,24 @@ public:
         if (entry.keys.dtype != dtype) raise(TQE_ERR_STATE, "pooled_attention: the cache holds %s, the step runs in %s", dtype_name(entry.keys.dtype), dtype_name(dtype));
         const StepContext::Table& table = c.tables.at((size_t)entry.group);
         const Tensor qkv = linear(c, x.x, w_qkv_, nullptr, dtype).t;
-        const Position::Tables tb = position_->tables();
-        Position::Tables vt;
+        Position::Tables tb, vt;
+        if (position_) tb = position_->tables();
         if (rotate_values_) vt = value_position_->tables();
         const bool turn = tb.style != STYLE_NONE;
-        const int max_pos = rotate_values_ ? (int)std::min(tb.cos.shape[0], vt.cos.shape[0]) : turn ? (int)tb.cos.shape[0] : 1 << 30;
+        const int style = rotate_values_ ? vt.style : tb.style;
+        const int max_pos = rotate_values_ && turn ? (int)std::min(tb.cos.shape[0], vt.cos.shape[0]) : rotate_values_ ? (int)vt.cos.shape[0] : turn ? (int)tb.cos.shape[0] : 1 << 30;
         const float* vcos = rotate_values_ ? (const float*)vt.cos.data : nullptr;
         const float* vsin = rotate_values_ ? (const float*)vt.sin.data : nullptr;
         Tensor q = c.alloc(dtype, {n, n_heads_, head_dim_});
         K::pooled_store(qkv.data, dtype, qk_norm_ ? (const float*)q_norm_->t.data : nullptr, qk_norm_ ? (const float*)k_norm_->t.data : nullptr, qk_norm_ ? 1 : 0, eps_,
-                        turn ? (const float*)tb.cos.data : nullptr, turn ? (const float*)tb.sin.data : nullptr, turn ? tb.rot_dim : 0, tb.style, vcos, vsin, max_pos,
+                        turn ? (const float*)tb.cos.data : nullptr, turn ? (const float*)tb.sin.data : nullptr, turn ? tb.rot_dim : 0, style, vcos, vsin, max_pos,
                         c.dev.tok_seq, c.dev.tok_pos, table.dev, table.width, entry.keys.data, entry.values.data, q.data, (int)n, n_heads_, n_kv_heads_, head_dim_,
                         value_dim_, pool_, c.stream);
         K::pool_blocks(entry.keys.data, entry.values.data, dtype, c.dev.seq_start, c.dev.seq_new, table.dev, table.width, c.n_seqs, c.max_new, pool_, n_kv_heads_,
                        head_dim_, value_dim_, c.stream);
         Tensor y = c.alloc(dtype, {n, (int64_t)n_heads_ * value_dim_});
         K::pooled_attention(q.data, entry.keys.data, entry.values.data, dtype, c.dev.tok_seq, c.dev.tok_pos, table.dev, table.width, window_, pool_, scale_,
-                            has_sink_ ? (const float*)sink_->t.data : nullptr, vcos, vsin, tb.style, max_pos, y.data, (int)n, n_heads_, n_kv_heads_, head_dim_,
+                            has_sink_ ? (const float*)sink_->t.data : nullptr, vcos, vsin, style, max_pos, y.data, (int)n, n_heads_, n_kv_heads_, head_dim_,
                             value_dim_, c.stream);
         return linear(c, y, w_o_, nullptr, dtype).t;
     }

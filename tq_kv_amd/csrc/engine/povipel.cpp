@@ -39,7 +39,7 @@ const Json& object_at(const Json& parent, const char* key, const std::string& wh
 
 void rot_typed(const Json& raw, const std::string& where, long long dim, Json& m) {
     KeyReader rot(object_at(raw, "rot", where), where + ".rot");
-    const long long dims = rot.integer("dims", 2);
+    const long long dims = rot.integer("dims", 0);
     if (dims % 2 || dims > dim) raise(TQE_ERR_CONFIG, "%s.rot: dims %lld must be even and at most dim %lld", where.c_str(), dims, dim);
     m.set("rot_base", rot.number("base", true));
     m.set("rot_dims", dims);
@@ -171,6 +171,7 @@ ModelSpec povipel_spec(const Json& c) {
     const Json& max_pos = c["max_positions"];
     const PartSpec norm = part("layer_norm", {{"size", width}, {"eps", eps}, {"tensor", ""}, {"bias_tensor", ".b"}});
     auto rotary = [&](const Json& base, const Json& dims, const char* style) {
+        if (dims.as_int() == 0) return Json();          // nothing is turned
         return part("rotary", {{"theta", base}, {"rot_dim", dims}, {"max_positions", max_pos}, {"style", style}}).to_json();
     };
     ModelSpec s;

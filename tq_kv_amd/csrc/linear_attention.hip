@@ -132,6 +132,128 @@ void linear_attention_kernel(LaArgs a, int rg_shift) {
     }
 }
 
+// The same with a block of the state per thread: RT neighbouring rows by four neighbouring columns, for heads whose sizes are multiples of
+// four.  A token costs a thread three 16-byte LDS reads per four rows (q, k and the decay) and one for its four values, for 4 RT state
+// elements; rows beyond the head's (the padding up to RG * RT) stay zero.
+template <typename T, int RT, int MODE>
+__global__ __launch_bounds__(LA_THREADS)
+void linear_attention_block_kernel(LaArgs a, int rg_shift, int cb) {
+    extern __shared__ float la_lds[];
+    const int d = a.d, dv = a.dv, H = a.H;
+    const int head = blockIdx.y, item = blockIdx.z;
+    const int RG = 1 << rg_shift, dpad = RG * RT;
+    const int rg = threadIdx.x & (RG - 1), cg = threadIdx.x >> rg_shift;
+    const int col0 = blockIdx.x * cb + cg * 4;
+    const bool col_ok = cg * 4 < cb && col0 < dv;
+    int row0, count;
+    if (MODE == LA_SCAN) { row0 = a.cu[item]; count = a.seq_new[item]; }
+    else { row0 = a.chunk_row0[item]; count = a.chunk_count[item]; }
+    if (count <= 0) return;
+    const size_t per_head = (size_t)d * dv;
+    float* sp = MODE == LA_SCAN ? a.state + (size_t)a.seq_slot[item] * a.state_stride + head * per_head
+                                : a.chunk_state + ((size_t)item * H + head) * per_head;
+    float S[RT][4], P[RT];
+#pragma unroll
+    for (int i = 0; i < RT; ++i) {
+        const int r = rg * RT + i;
+#pragma unroll
+        for (int c = 0; c < 4; ++c) S[i][c] = (MODE != LA_LOCAL && r < d && col_ok) ? sp[(size_t)r * dv + col0 + c] : 0.f;
+        P[i] = 1.f;
+    }
+    float* lq = la_lds;
+    float* lk = lq + LA_TB * dpad;
+    float* ld = lk + LA_TB * dpad;
+    float* lv = ld + LA_TB * dpad;
+    const T* qb = (const T*)a.q + (size_t)head * d;
+    const T* kb = (const T*)a.k + (size_t)head * d;
+    const T* vb = (const T*)a.v + (size_t)head * dv;
+    const int half = a.rot_dim / 2;
+    for (int t0 = 0; t0 < count; t0 += LA_TB) {
+        const int nt = min(LA_TB, count - t0);
+        __syncthreads();
+        for (int e = threadIdx.x; e < nt * dpad; e += blockDim.x) {
+            const int tt = e / dpad, i = e - tt * dpad;
+            float qv = 0.f, kv = 0.f, al = 0.f;
+            if (i < d) {
+                const long long row = row0 + t0 + tt;
+                const T* qr = qb + row * a.stride;
+                const T* kr = kb + row * a.stride;
+                qv = to_float(qr[i]);
+                kv = to_float(kr[i]);
+                if (a.cos && i < a.rot_dim) {
+                    bool first;
+                    int pi, ai;
+                    if (a.style == LA_STYLE_HALVES) { first = i < half; pi = first ? i + half : i - half; ai = first ? i : i - half; }
+                    else { first = !(i & 1); pi = i ^ 1; ai = i >> 1; }
+                    const int pos = min(a.tok_pos[row], a.max_pos - 1);
+                    const float c = a.cos[(size_t)pos * half + ai], s = a.sin[(size_t)pos * half + ai];
+                    const float qp = to_float(qr[pi]), kp = to_float(kr[pi]);
+                    qv = first ? qv * c - qp * s : qv * c + qp * s;
+                    kv = first ? kv * c - kp * s : kv * c + kp * s;
+                }
+                qv *= a.q_scale;
+                kv *= a.k_scale;
+                if (a.z) {
+                    const float zz = a.z[row * a.z_stride + (size_t)head * d + i] + a.z_bias[(size_t)head * d + i];
+                    const float ls = fminf(zz, 0.f) - log1pf(expf(-fabsf(zz)));
+                    al = expf(ls * a.inv_tau);
+                } else al = a.head_decay[head];
+            }
+            lq[e] = qv;
+            lk[e] = kv;
+            ld[e] = al;
+        }
+        for (int e = threadIdx.x; e < nt * cb; e += blockDim.x) {
+            const int tt = e / cb, c = e - tt * cb, col = blockIdx.x * cb + c;
+            lv[e] = col < dv ? to_float(vb[(row0 + t0 + tt) * a.stride + col]) : 0.f;
+        }
+        __syncthreads();
+        if (cg * 4 < cb) {
+            for (int tt = 0; tt < nt; ++tt) {
+                const float4 vv = *reinterpret_cast<const float4*>(lv + tt * cb + cg * 4);
+                const float v4[4] = {vv.x, vv.y, vv.z, vv.w};
+                float o[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                for (int i = 0; i < RT; i += 4) {
+                    const float4 q4 = *reinterpret_cast<const float4*>(lq + tt * dpad + rg * RT + i);
+                    const float4 k4 = *reinterpret_cast<const float4*>(lk + tt * dpad + rg * RT + i);
+                    const float4 a4 = *reinterpret_cast<const float4*>(ld + tt * dpad + rg * RT + i);
+                    const float qq[4] = {q4.x, q4.y, q4.z, q4.w}, kk[4] = {k4.x, k4.y, k4.z, k4.w}, aa[4] = {a4.x, a4.y, a4.z, a4.w};
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) {
+#pragma unroll
+                        for (int c = 0; c < 4; ++c) {
+                            S[i + j][c] = fmaf(aa[j], S[i + j][c], kk[j] * v4[c]);
+                            o[c] = fmaf(S[i + j][c], qq[j], o[c]);
+                        }
+                        if (MODE == LA_LOCAL) P[i + j] *= aa[j];
+                    }
+                }
+                if (MODE != LA_LOCAL) {
+#pragma unroll
+                    for (int c = 0; c < 4; ++c)
+                        for (int m = RG >> 1; m > 0; m >>= 1) o[c] += __shfl_xor(o[c], m, TQK_WAVE);
+                    if (rg == 0 && col_ok) {
+                        float* dst = a.out + ((size_t)(row0 + t0 + tt) * H + head) * dv + col0;
+#pragma unroll
+                        for (int c = 0; c < 4; ++c) dst[c] = o[c];
+                    }
+                }
+            }
+        }
+    }
+    if (MODE == LA_APPLY) return;
+#pragma unroll
+    for (int i = 0; i < RT; ++i) {
+        const int r = rg * RT + i;
+        if (r < d && col_ok) {
+#pragma unroll
+            for (int c = 0; c < 4; ++c) sp[(size_t)r * dv + col0 + c] = S[i][c];
+        }
+        if (MODE == LA_LOCAL && r < d && col0 == 0 && col_ok) a.chunk_decay[((size_t)item * H + head) * d + r] = P[i];
+    }
+}
+
 // out[t, h, j] = o[t, h, j] / sqrt(mean_j o[t, h]^2 + eps) * w[j] * silu(gate[t, h * dv + j]); a wave per (token, head)
 template <typename TG, typename TO>
 __global__ __launch_bounds__(256)
@@ -175,6 +297,33 @@ extern "C" int tqk_linear_attention(const void* q, const void* k, const void* v,
     TQK_REQUIRE(!cos || (sin && tok_pos && rot_dim > 0 && rot_dim % 2 == 0 && rot_dim <= d && max_pos > 0 && (style == LA_STYLE_HALVES || style == LA_STYLE_PAIRS)),
                 "tqk_linear_attention: bad rotation");
     if (n_items == 0) return 0;
+    LaArgs a = {q, k, v, stride, z, z_stride, z_bias, inv_tau, head_decay, q_scale, k_scale, cos, sin, rot_dim, style, max_pos, tok_pos, state, state_stride,
+                cu, seq_new, seq_slot, chunk_row0, chunk_count, chunk_state, chunk_decay, out, heads, d, dv};
+    hipStream_t s = (hipStream_t)stream;
+    if (d % 4 == 0 && dv % 4 == 0 && dv >= 16 && (((uintptr_t)out) & 15) == 0) {
+        // a thread holds rt rows by four columns: rt = 16 where the head has the rows for it, and as many row groups as cover the head
+        const int rt = d >= 64 ? 16 : d >= 32 ? 8 : 4;
+        int shift = 0;
+        while ((rt << shift) < d) ++shift;
+        if ((1 << shift) <= TQK_WAVE) {
+            const int groups = LA_THREADS >> shift;                        // column groups a block has threads for
+            const int cb = 4 * (((dv + 3) / 4 < groups) ? (dv + 3) / 4 : groups);
+            int threads = ((cb / 4) << shift);
+            threads = (threads + TQK_WAVE - 1) / TQK_WAVE * TQK_WAVE;
+            dim3 bgrid((dv + cb - 1) / cb, heads, n_items);
+            const size_t blds = (size_t)LA_TB * (3 * (size_t)(rt << shift) + cb) * sizeof(float);
+#define TQK_LAB(T, RT, MODE) linear_attention_block_kernel<T, RT, MODE><<<bgrid, threads, blds, s>>>(a, shift, cb)
+#define TQK_LAB_MODE(T, RT) do { if (mode == LA_SCAN) TQK_LAB(T, RT, LA_SCAN); else if (mode == LA_LOCAL) TQK_LAB(T, RT, LA_LOCAL); else TQK_LAB(T, RT, LA_APPLY); } while (0)
+#define TQK_LAB_ROWS(T) do { if (rt == 16) TQK_LAB_MODE(T, 16); else if (rt == 8) TQK_LAB_MODE(T, 8); else TQK_LAB_MODE(T, 4); } while (0)
+            if (act_dtype == TQK_F32) TQK_LAB_ROWS(float);
+            else if (act_dtype == TQK_BF16) TQK_LAB_ROWS(bf16_t);
+            else return tqk_fail("tqk_linear_attention: unknown dtype %d", act_dtype);
+#undef TQK_LAB_ROWS
+#undef TQK_LAB_MODE
+#undef TQK_LAB
+            return tqk_check_launch("tqk_linear_attention");
+        }
+    }
     // the widest slab of columns (a power of two up to 128, no wider than the head needs) whose threads hold at most 64 rows each
     int cb = 16;
     while (cb < 128 && cb < dv) cb *= 2;
@@ -184,11 +333,8 @@ extern "C" int tqk_linear_attention(const void* q, const void* k, const void* v,
     while ((1 << rg_shift) < rg) ++rg_shift;
     const int rows = (d + rg - 1) / rg;
     TQK_REQUIRE(rows <= 64, "tqk_linear_attention: %d rows a thread", rows);
-    LaArgs a = {q, k, v, stride, z, z_stride, z_bias, inv_tau, head_decay, q_scale, k_scale, cos, sin, rot_dim, style, max_pos, tok_pos, state, state_stride,
-                cu, seq_new, seq_slot, chunk_row0, chunk_count, chunk_state, chunk_decay, out, heads, d, dv};
     dim3 grid((dv + cb - 1) / cb, heads, n_items);
     const size_t lds = (size_t)3 * LA_TB * d * sizeof(float);
-    hipStream_t s = (hipStream_t)stream;
 #define TQK_LA(T, RT, MODE) linear_attention_kernel<T, RT, MODE><<<grid, LA_THREADS, lds, s>>>(a, rg_shift)
 #define TQK_LA_MODE(T, RT) do { if (mode == LA_SCAN) TQK_LA(T, RT, LA_SCAN); else if (mode == LA_LOCAL) TQK_LA(T, RT, LA_LOCAL); else TQK_LA(T, RT, LA_APPLY); } while (0)
 #define TQK_LA_ROWS(T) do { if (rows <= 1) TQK_LA_MODE(T, 1); else if (rows <= 2) TQK_LA_MODE(T, 2); else if (rows <= 4) TQK_LA_MODE(T, 4); \

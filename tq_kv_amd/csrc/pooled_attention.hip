@@ -197,7 +197,7 @@ extern "C" int tqk_pooled_store(const void* qkv, int dtype, const float* q_weigh
                                 int heads, int kv_heads, int d, int dv, int pool, void* stream) {
     TQK_REQUIRE(qkv && tok_seq && tok_pos && table && keys && values && q_out, "tqk_pooled_store: null pointer");
     TQK_REQUIRE(n_tokens >= 0 && heads > 0 && kv_heads > 0 && d > 0 && dv > 0 && pool > 0 && width > 0, "tqk_pooled_store: bad sizes");
-    TQK_REQUIRE(style == PA_STYLE_NONE || (cos && sin && rot_dim > 0 && rot_dim % 2 == 0 && rot_dim <= d && max_pos > 0), "tqk_pooled_store: bad rotation");
+    TQK_REQUIRE(style == PA_STYLE_NONE || rot_dim == 0 || (cos && sin && rot_dim > 0 && rot_dim % 2 == 0 && rot_dim <= d && max_pos > 0), "tqk_pooled_store: bad rotation");
     TQK_REQUIRE(!vcos || (vsin && dv % 2 == 0 && style != PA_STYLE_NONE), "tqk_pooled_store: values are turned in the layout of the keys, over an even number of elements");
     if (n_tokens == 0) return 0;
     const long long items = (long long)n_tokens * (heads + 2 * kv_heads), blocks = (items + 3) / 4;

@@ -14,7 +14,7 @@
 #include "common.h"
 #include "tq_kernels.h"
 
-#define STREAMS_MAX 8
+#define STREAMS_MAX 16
 
 __global__ __launch_bounds__(256)
 void streams_fill_kernel(const float* __restrict__ h, float* __restrict__ X, int S, int W) {
@@ -34,7 +34,7 @@ void streams_step_kernel(float* __restrict__ X, int S, const TY* __restrict__ y,
     __shared__ float scratch[4];
     __shared__ float s_mix[STREAMS_MAX * STREAMS_MAX], s_out[STREAMS_MAX], s_in[STREAMS_MAX];
     const size_t t = blockIdx.x;
-    if (threadIdx.x < S * S && y) s_mix[threadIdx.x] = mix[threadIdx.x];
+    for (int i = threadIdx.x; i < S * S && y; i += blockDim.x) s_mix[i] = mix[i];
     if (threadIdx.x < S) {
         if (y) s_out[threadIdx.x] = outw[threadIdx.x];
         if (in) s_in[threadIdx.x] = in[threadIdx.x];
