@@ -18,7 +18,7 @@ import time
 
 HERE = os.path.dirname(os.path.abspath(__file__))
 SOURCES = ["host.cpp", "elementwise.hip", "gemm_generic.hip", "attention_generic.hip", "sampling.hip",
-           "attention_decode.hip", "attention_prefill.hip", "skinny_fused.hip", "mid_product.hip", "random_init.hip", "utility.hip", "probe.hip", "latent.hip", "moe.hip", "grouped.hip", "stream_ops.hip", "attention_masked.hip", "attention_masked_mfma.hip", "recurrent.hip", "streams.hip", "linear_attention.hip", "pooled_attention.hip"]
+           "attention_decode.hip", "attention_prefill.hip", "skinny_fused.hip", "mid_product.hip", "random_init.hip", "utility.hip", "probe.hip", "latent.hip", "moe.hip", "grouped.hip", "stream_ops.hip", "attention_masked.hip", "attention_masked_mfma.hip", "recurrent.hip", "streams.hip", "linear_attention.hip", "pooled_attention.hip", "pooled_attention_mfma.hip"]
 HEADERS = ["common.h", "tq_kernels.h", "tq_no_alloc.h"]
 # the engine: host code only (config, weights, parts, model, cache, step, loop), built with the host compiler into a
 # library of its own that reaches the GPU through the HIP runtime, hipBLASLt and the kernel library above

@@ -123,6 +123,10 @@ TQ_KERNEL(pooled_store, cptr, int, cf32, cf32, int, float, cf32, cf32, int, int,
 TQ_KERNEL(pool_blocks, void*, void*, int, ci32, ci32, ci32, int, int, int, int, int, int, int, void*);
 TQ_KERNEL(pooled_attention, cptr, cptr, cptr, int, ci32, ci32, ci32, int, int, int, float, cf32, cf32, cf32, int, int, void*, int, int, int, int, int,
           void*);
+TQ_QUERY(int, pooled_attention_tiles_supported, int, int);
+TQ_QUERY(int, pooled_attention_tile, int, int);
+TQ_KERNEL(pooled_attention_tiles, cptr, cptr, cptr, ci32, ci32, int, int, int, float, cf32, cf32, cf32, int, int, ci32, ci32, ci32, int, int, void*, int, int,
+          int, int, void*);
 TQ_KERNEL(normed_pair_sum, cptr, cptr, int, cf32, cf32, float, float, void*, int, int, int, void*);
 TQ_QUERY(int, argmax_scratch_floats, int, int);
 TQ_KERNEL(argmax, cf32, int, int, int32_t*, float*, void*);

@@ -156,6 +156,17 @@ public:
         K::pool_blocks(entry.keys.data, entry.values.data, dtype, c.dev.seq_start, c.dev.seq_new, table.dev, table.width, c.n_seqs, c.max_new, pool_, n_kv_heads_,
                        head_dim_, value_dim_, c.stream);
         Tensor y = c.alloc(dtype, {n, (int64_t)n_heads_ * value_dim_});
+        // bfloat16 steps that bring several tokens of a sequence: tiles of consecutive queries on the matrix cores, where the heads' sizes
+        // allow; steps of one token a sequence, the 32-bit path and other sizes: the plain kernel, a wave per (row, head)
+        if (dtype == BF16 && !c.all_decode && !c.capturing && policy().prefill_mfma && !null_device() &&
+            K::pooled_attention_tiles_supported.raw(head_dim_, value_dim_)) {
+            const int tile = K::pooled_attention_tile.raw(n_heads_, n_kv_heads_);
+            const Tiles t = c.query_tiles(tile);
+            K::pooled_attention_tiles(q.data, entry.keys.data, entry.values.data, c.dev.tok_pos, table.dev, table.width, window_, pool_, scale_,
+                                      has_sink_ ? (const float*)sink_->t.data : nullptr, vcos, vsin, style, max_pos, t.seq, t.tok0, t.count, t.n, tile, y.data,
+                                      n_heads_, n_kv_heads_, head_dim_, value_dim_, c.stream);
+            return linear(c, y, w_o_, nullptr, dtype).t;
+        }
         K::pooled_attention(q.data, entry.keys.data, entry.values.data, dtype, c.dev.tok_seq, c.dev.tok_pos, table.dev, table.width, window_, pool_, scale_,
                             has_sink_ ? (const float*)sink_->t.data : nullptr, vcos, vsin, style, max_pos, y.data, (int)n, n_heads_, n_kv_heads_, head_dim_,
                             value_dim_, c.stream);

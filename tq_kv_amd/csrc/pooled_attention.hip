@@ -15,7 +15,8 @@
 //                         elements (optional); q out, k and v into the pages
 //   tqk_pool_blocks       the means of the blocks that the step completes
 //   tqk_pooled_attention  a wave per (row, head): blocks first, then the window's positions, 64 at a time: a lane a key for the scores,
-//                         a lane an output element (and every 64th after it) for the values; softmax in float32
+//                         a lane an output element (and every 64th after it) for the values; softmax in float32.  Heads of 8 n key
+//                         elements and 2 n values: several waves per (row, head) and wider loads
 #include "common.h"
 #include "tq_kernels.h"
 
@@ -188,6 +189,115 @@ void pooled_attention_kernel(const T* __restrict__ q, const T* __restrict__ keys
         out[((size_t)r * H + h) * dv + i] = from_float<T>(pa_turned(get, i, dv, vcos ? style : PA_STYLE_NONE, vcos, vsin, tpos, -1.f));
 }
 
+// The same for heads whose keys are multiples of 8 elements and whose values are an even number: a block of W waves per (row, head), the
+// waves taking the batches of 64 keys in turn and meeting in LDS in the order of the waves; a key's row is read 16 bytes at a time, a
+// lane owns two neighbouring output elements (and the two 128 further on).
+template <typename T, int W>
+__global__ __launch_bounds__(W * TQK_WAVE)
+void pooled_attention_rows_kernel(const T* __restrict__ q, const T* __restrict__ keys, const T* __restrict__ values, const int32_t* __restrict__ row_seq,
+                                  const int32_t* __restrict__ row_pos, const int32_t* __restrict__ table, int width, int window, int pool, float scale,
+                                  const float* __restrict__ sink, const float* __restrict__ vcos, const float* __restrict__ vsin, int style, int max_pos,
+                                  T* __restrict__ out, int H, int G, int d, int dv, int page_rows) {
+    __shared__ __attribute__((aligned(16))) float q_lds[PA_MAX_DIM];
+    __shared__ float o_lds[W][PA_MAX_DIM];
+    __shared__ float ml_lds[W][2];
+    const int wave = threadIdx.x / TQK_WAVE, lane = threadIdx.x % TQK_WAVE;
+    const long long item = blockIdx.x;
+    const long long r = item / H;
+    const int h = (int)(item % H), g = h / (H / G);
+    const int pos = row_pos[r];
+    const int32_t* pages = table + (size_t)row_seq[r] * width;
+    for (int i = threadIdx.x; i < d; i += W * TQK_WAVE) q_lds[i] = to_float(q[((size_t)r * H + h) * d + i]) * scale;
+    __syncthreads();
+    const int lo = max(0, pos - window + 1);
+    const int n_blocks = pos - window + 1 >= pool ? (pos - window + 1) / pool : 0;
+    const int n_all = n_blocks + (pos - lo + 1);
+    float m = -INFINITY, l = 0.f;
+    float acc[2][2] = {{0.f, 0.f}, {0.f, 0.f}};
+    for (int n0 = wave * TQK_WAVE; n0 < n_all; n0 += W * TQK_WAVE) {
+        const int n = n0 + lane;
+        long long row = -1;
+        if (n < n_all) {
+            int page, in_page;
+            if (n < n_blocks) { page = pages[(n * pool + pool - 1) / TQK_PAGE]; in_page = pa_pooled_row(n, pool); }
+            else { const int j = lo + (n - n_blocks); page = pages[j / TQK_PAGE]; in_page = j % TQK_PAGE; }
+            row = ((long long)page * G + g) * page_rows + in_page;
+        }
+        float s = -INFINITY;
+        if (row >= 0) {
+            const T* kr = keys + (size_t)row * d;
+            float d0 = 0.f, d1 = 0.f;
+            for (int i = 0; i < d; i += 8) {
+                const float4 qa = *reinterpret_cast<const float4*>(q_lds + i), qb = *reinterpret_cast<const float4*>(q_lds + i + 4);
+                float k8[8];
+                if (sizeof(T) == 2) {
+                    const uint4 kv = *reinterpret_cast<const uint4*>(kr + i);
+                    const uint32_t w4[4] = {kv.x, kv.y, kv.z, kv.w};
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) { k8[2 * j] = __uint_as_float(w4[j] << 16); k8[2 * j + 1] = __uint_as_float(w4[j] & 0xffff0000u); }
+                } else {
+                    const float4 ka = *reinterpret_cast<const float4*>(kr + i), kb = *reinterpret_cast<const float4*>(kr + i + 4);
+                    k8[0] = ka.x; k8[1] = ka.y; k8[2] = ka.z; k8[3] = ka.w; k8[4] = kb.x; k8[5] = kb.y; k8[6] = kb.z; k8[7] = kb.w;
+                }
+                d0 = fmaf(qa.x, k8[0], d0); d1 = fmaf(qa.y, k8[1], d1); d0 = fmaf(qa.z, k8[2], d0); d1 = fmaf(qa.w, k8[3], d1);
+                d0 = fmaf(qb.x, k8[4], d0); d1 = fmaf(qb.y, k8[5], d1); d0 = fmaf(qb.z, k8[6], d0); d1 = fmaf(qb.w, k8[7], d1);
+            }
+            s = d0 + d1;
+        }
+        const float m_new = fmaxf(m, wave_max(s));
+        const float corr = expf(m - m_new);
+        const float p = row >= 0 ? expf(s - m_new) : 0.f;
+        l = l * corr + wave_sum(p);
+        m = m_new;
+        acc[0][0] *= corr; acc[0][1] *= corr; acc[1][0] *= corr; acc[1][1] *= corr;
+        const int n_here = min(TQK_WAVE, n_all - n0);
+        for (int k = 0; k < n_here; ++k) {
+            const float pk = __shfl(p, k, TQK_WAVE);
+            const long long rk = __shfl(row, k, TQK_WAVE);
+            const T* vr = values + (size_t)rk * dv;
+#pragma unroll
+            for (int c = 0; c < 2; ++c) {
+                const int i = c * 2 * TQK_WAVE + 2 * lane;
+                if (i < dv) {
+                    float v0, v1;
+                    if (sizeof(T) == 2) { const uint32_t vv = *reinterpret_cast<const uint32_t*>(vr + i); v0 = __uint_as_float(vv << 16); v1 = __uint_as_float(vv & 0xffff0000u); }
+                    else { const float2 vv = *reinterpret_cast<const float2*>(vr + i); v0 = vv.x; v1 = vv.y; }
+                    acc[c][0] = fmaf(pk, v0, acc[c][0]);
+                    acc[c][1] = fmaf(pk, v1, acc[c][1]);
+                }
+            }
+        }
+    }
+    // the waves meet: every one leaves its maximum, its sum and its part of the output; the first adds them up in their order
+    if (lane == 0) { ml_lds[wave][0] = m; ml_lds[wave][1] = l; }
+#pragma unroll
+    for (int c = 0; c < 2; ++c) {
+        const int i = c * 2 * TQK_WAVE + 2 * lane;
+        if (i < dv) { o_lds[wave][i] = acc[c][0]; o_lds[wave][i + 1] = acc[c][1]; }
+    }
+    __syncthreads();
+    if (wave != 0) return;
+    float mt = sink ? sink[h] : -INFINITY;
+    for (int w = 0; w < W; ++w) mt = fmaxf(mt, ml_lds[w][0]);
+    float lt = sink ? expf(sink[h] - mt) : 0.f;
+    float f[W];
+    for (int w = 0; w < W; ++w) {
+        f[w] = ml_lds[w][0] == -INFINITY ? 0.f : expf(ml_lds[w][0] - mt);
+        lt = fmaf(ml_lds[w][1], f[w], lt);
+    }
+    const float inv = 1.f / lt;
+    for (int i = lane; i < dv; i += TQK_WAVE) {
+        float v = 0.f;
+        for (int w = 0; w < W; ++w) v = fmaf(o_lds[w][i], f[w], v);
+        q_lds[i] = v * inv;                 // (the query is no longer needed)
+    }
+    __builtin_amdgcn_wave_barrier();
+    auto get = [&](int i) { return q_lds[i]; };
+    const int tpos = min(pos, max_pos - 1);
+    for (int i = lane; i < dv; i += TQK_WAVE)
+        out[((size_t)r * H + h) * dv + i] = from_float<T>(pa_turned(get, i, dv, vcos ? style : PA_STYLE_NONE, vcos, vsin, tpos, -1.f));
+}
+
 extern "C" int tqk_pooled_attention_max_dim(void) { return PA_MAX_DIM; }
 extern "C" int tqk_pooled_rows(int pool) { return pool > 0 ? (TQK_PAGE + pool - 1) / pool : 0; }
 
@@ -237,9 +347,22 @@ extern "C" int tqk_pooled_attention(const void* q, const void* keys, const void*
     TQK_REQUIRE(!vcos || (vsin && dv % 2 == 0 && max_pos > 0 && (style == PA_STYLE_HALVES || style == PA_STYLE_PAIRS)), "tqk_pooled_attention: bad rotation of the values");
     if (n_rows == 0) return 0;
     const long long items = (long long)n_rows * heads, blocks = (items + 3) / 4;
-    TQK_REQUIRE(blocks <= 0x7fffffff, "tqk_pooled_attention: too many rows");
+    TQK_REQUIRE(items <= 0x7fffffff, "tqk_pooled_attention: too many rows");
     const int page_rows = TQK_PAGE + tqk_pooled_rows(pool);
     hipStream_t s = (hipStream_t)stream;
+    const int esize = dtype == TQK_BF16 ? 2 : 4;
+    if (d % 8 == 0 && dv % 2 == 0 && (((uintptr_t)keys | (uintptr_t)values) & 15) == 0 && (dtype == TQK_BF16 || dtype == TQK_F32) && ((size_t)dv * esize) % 4 == 0) {
+        // 32-bit steps keep one shape whatever the step holds (the order of the sums is then the position's alone); others deal a row's
+        // keys out to more waves the fewer rows there are
+#define TQK_PAR(T, W) pooled_attention_rows_kernel<T, W><<<(unsigned)items, W * TQK_WAVE, 0, s>>>((const T*)q, (const T*)keys, (const T*)values, row_seq, row_pos, table, \
+        width, window, pool, scale, sink, vcos, vsin, style, max_pos, (T*)out, heads, kv_heads, d, dv, page_rows)
+        if (dtype == TQK_F32) TQK_PAR(float, 4);
+        else if (items >= 4096) TQK_PAR(bf16_t, 1);
+        else if (items >= 1024) TQK_PAR(bf16_t, 4);
+        else TQK_PAR(bf16_t, 8);
+#undef TQK_PAR
+        return tqk_check_launch("tqk_pooled_attention");
+    }
 #define TQK_PA(T) pooled_attention_kernel<T><<<(unsigned)blocks, 256, 0, s>>>((const T*)q, (const T*)keys, (const T*)values, row_seq, row_pos, table, width, window, \
         pool, scale, sink, vcos, vsin, style, max_pos, (T*)out, items, heads, kv_heads, d, dv, page_rows)
     if (dtype == TQK_F32) TQK_PA(float);

@@ -25,7 +25,8 @@ void streams_fill_kernel(const float* __restrict__ h, float* __restrict__ X, int
     }
 }
 
-template <typename TY, typename TN>
+// SMAX: the most copies this instance takes (the loops over the copies are unrolled up to it)
+template <typename TY, typename TN, int SMAX>
 __global__ __launch_bounds__(256)
 void streams_step_kernel(float* __restrict__ X, int S, const TY* __restrict__ y, const float* __restrict__ mix, const float* __restrict__ outw,
                          const float* __restrict__ in, const float* __restrict__ nw, const float* __restrict__ nb, float eps,
@@ -43,18 +44,18 @@ void streams_step_kernel(float* __restrict__ X, int S, const TY* __restrict__ y,
     float* xr = X + t * S * W;
     float sum = 0.f;
     for (int e = threadIdx.x; e < W; e += blockDim.x) {
-        float x[STREAMS_MAX];
+        float x[SMAX];
 #pragma unroll
-        for (int s = 0; s < STREAMS_MAX; ++s) x[s] = s < S ? xr[(size_t)s * W + e] : 0.f;
+        for (int s = 0; s < SMAX; ++s) x[s] = s < S ? xr[(size_t)s * W + e] : 0.f;
         if (y) {
             const float yv = to_float(y[t * W + e]);
-            float nx[STREAMS_MAX];
+            float nx[SMAX];
 #pragma unroll
-            for (int r = 0; r < STREAMS_MAX; ++r) {
+            for (int r = 0; r < SMAX; ++r) {
                 float acc = 0.f;
                 if (r < S) {
 #pragma unroll
-                    for (int s = 0; s < STREAMS_MAX; ++s)
+                    for (int s = 0; s < SMAX; ++s)
                         if (s < S) acc = fmaf(s_mix[s * S + r], x[s], acc);
                     acc = fmaf(s_out[r], yv, acc);
                     xr[(size_t)r * W + e] = acc;
@@ -62,12 +63,12 @@ void streams_step_kernel(float* __restrict__ X, int S, const TY* __restrict__ y,
                 nx[r] = acc;
             }
 #pragma unroll
-            for (int s = 0; s < STREAMS_MAX; ++s) x[s] = nx[s];
+            for (int s = 0; s < SMAX; ++s) x[s] = nx[s];
         }
         if (in) {
             float u = 0.f;
 #pragma unroll
-            for (int s = 0; s < STREAMS_MAX; ++s)
+            for (int s = 0; s < SMAX; ++s)
                 if (s < S) u = fmaf(s_in[s], x[s], u);
             row_u[e] = u;
             sum += u;
@@ -153,7 +154,9 @@ extern "C" int tqk_streams_step(float* X, int n_streams, const void* y, int y_dt
     if (n_tokens == 0 || (!y && !in_w)) return 0;
     hipStream_t s = (hipStream_t)stream;
     const size_t lds = (size_t)width * sizeof(float);
-#define TQK_SS(TY, TN) streams_step_kernel<TY, TN><<<n_tokens, 256, lds, s>>>(X, n_streams, (const TY*)y, mix, out_w, in_w, norm_w, norm_b, eps, u_out, (TN*)n_out, width)
+#define TQK_SS_N(TY, TN, SMAX) streams_step_kernel<TY, TN, SMAX><<<n_tokens, 256, lds, s>>>(X, n_streams, (const TY*)y, mix, out_w, in_w, norm_w, norm_b, eps, u_out, (TN*)n_out, width)
+#define TQK_SS(TY, TN) do { if (n_streams <= 1) TQK_SS_N(TY, TN, 1); else if (n_streams <= 2) TQK_SS_N(TY, TN, 2); else if (n_streams <= 4) TQK_SS_N(TY, TN, 4); \
+        else if (n_streams <= 8) TQK_SS_N(TY, TN, 8); else TQK_SS_N(TY, TN, STREAMS_MAX); } while (0)
     const int yd = y ? y_dtype : TQK_F32, nd = n_out ? n_dtype : TQK_F32;
     if (yd == TQK_F32 && nd == TQK_F32) TQK_SS(float, float);
     else if (yd == TQK_F32 && nd == TQK_BF16) TQK_SS(float, bf16_t);
@@ -161,6 +164,7 @@ extern "C" int tqk_streams_step(float* X, int n_streams, const void* y, int y_dt
     else if (yd == TQK_BF16 && nd == TQK_BF16) TQK_SS(bf16_t, bf16_t);
     else return tqk_fail("tqk_streams_step: unknown dtypes %d, %d", y_dtype, n_dtype);
 #undef TQK_SS
+#undef TQK_SS_N
     return tqk_check_launch("tqk_streams_step");
 }
 

@@ -477,6 +477,15 @@ int tqk_pooled_attention(const void* q, const void* keys, const void* values, in
                          const int32_t* table, int width, int window, int pool, float scale, const float* sink, const float* vcos,
                          const float* vsin, int style, int max_pos, void* out, int n_rows, int heads, int kv_heads, int d, int dv,
                          void* stream);
+/* The same attention on the matrix cores for steps that bring several tokens of a sequence (pooled_attention_mfma.hip; bfloat16, head
+ * sizes that are multiples of 32 up to 256): tiles of tqk_pooled_attention_tile(heads, kv_heads) consecutive queries of one sequence
+ * (sequence of the step, first packed token, number of queries). */
+int tqk_pooled_attention_tiles_supported(int d, int dv);
+int tqk_pooled_attention_tile(int heads, int kv_heads);
+int tqk_pooled_attention_tiles(const void* q, const void* keys, const void* values, const int32_t* tok_pos, const int32_t* table, int width,
+                               int window, int pool, float scale, const float* sink, const float* vcos, const float* vsin, int style,
+                               int max_pos, const int32_t* tile_seq, const int32_t* tile_tok0, const int32_t* tile_count, int n_tiles,
+                               int tile_queries, void* out, int heads, int kv_heads, int d, int dv, void* stream);
 /* out[t] = c (x[t] / rms(x[t]) wx + y[t] / rms(y[t]) wy) over rows of `width` elements (streams.hip) */
 int tqk_normed_pair_sum(const void* x, const void* y, int dtype, const float* wx, const float* wy, float eps, float c, void* out, int out_dtype,
                         int n_tokens, int width, void* stream);
