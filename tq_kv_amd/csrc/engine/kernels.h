@@ -108,7 +108,7 @@ TQ_KERNEL(attention_masked, cptr, cptr, cptr, int, ci32, ci32, ci32, int, int, i
           int, void*);
 TQ_QUERY(int, streams_max);
 TQ_KERNEL(streams_fill, cf32, float*, int, int, int, void*);
-TQ_KERNEL(streams_step, float*, int, cptr, int, cf32, cf32, cf32, cf32, cf32, float, float*, void*, int, int, int, void*);
+TQ_KERNEL(streams_step, float*, int, cptr, int, cf32, cf32, cf32, cf32, cf32, float, float*, void*, int, int, int, int, void*);
 TQ_KERNEL(add_layer_norm, float*, cptr, int, ci32, int, cf32, cf32, float, void*, int, int, int, void*);
 TQ_KERNEL(token_shift, cf32, cf32, float*, long long, ci32, ci32, ci32, ci32, void*, int, int, int, int, void*);
 TQ_KERNEL(shift_remember, cf32, float*, long long, ci32, ci32, ci32, int, int, void*);

@@ -252,7 +252,7 @@ public:
         if (last) {
             // nothing but the head reads the stream after this block: the copies' sum, with the last update on its way
             K::streams_step((float*)stream->copies.data, S, stream->pending.t.data, stream->pending.t.dtype, stream->copies_mix, stream->copies_out,
-                            (const float*)ones_->t.data, nullptr, nullptr, 0.f, (float*)stream->h.data, nullptr, 0, (int)n, (int)hidden_, c.stream);
+                            (const float*)ones_->t.data, nullptr, nullptr, 0.f, (float*)stream->h.data, nullptr, 0, (int)n, (int)hidden_, wide(c), c.stream);
             stream->pending = Pending();
             stream->copies_mix = stream->copies_out = nullptr;
         }
@@ -261,6 +261,9 @@ public:
 
 private:
     struct Role { std::string role, prefix; std::shared_ptr<Part> part; };
+
+    // bfloat16 steps of few tokens give a row more threads; 32-bit steps keep one order of a row's sums whatever the step holds
+    static int wide(const StepContext& c) { return c.act_dtype == BF16 && c.n_tokens <= 64 ? 1 : 0; }
 
     // what sublayer q reads: the pending update of the copies, then the norm of their weighted sum
     Tensor read(StepContext& c, Stream& s, int q, int dtype) {
@@ -273,12 +276,12 @@ private:
         const LayerNorm* ln = dynamic_cast<const LayerNorm*>(norm);
         if (ln) {
             K::streams_step((float*)s.copies.data, streams_, pending ? s.pending.t.data : nullptr, pending ? s.pending.t.dtype : 0, s.copies_mix, s.copies_out,
-                            (const float*)in_[q]->t.data, ln->weight(), ln->bias(), ln->eps(), nullptr, out.data, out.dtype, (int)n, (int)hidden_, c.stream);
+                            (const float*)in_[q]->t.data, ln->weight(), ln->bias(), ln->eps(), nullptr, out.data, out.dtype, (int)n, (int)hidden_, wide(c), c.stream);
         } else {
             // another norm: the weighted sum from the kernel, the norm as a step of its own
             Tensor u = c.alloc(F32, {n, hidden_});
             K::streams_step((float*)s.copies.data, streams_, pending ? s.pending.t.data : nullptr, pending ? s.pending.t.dtype : 0, s.copies_mix, s.copies_out,
-                            (const float*)in_[q]->t.data, nullptr, nullptr, 0.f, (float*)u.data, nullptr, 0, (int)n, (int)hidden_, c.stream);
+                            (const float*)in_[q]->t.data, nullptr, nullptr, 0.f, (float*)u.data, nullptr, 0, (int)n, (int)hidden_, wide(c), c.stream);
             norm->forward(c, u, out);
         }
         s.pending = Pending();

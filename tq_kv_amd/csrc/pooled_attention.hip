@@ -227,6 +227,7 @@ void pooled_attention_rows_kernel(const T* __restrict__ q, const T* __restrict__
         if (row >= 0) {
             const T* kr = keys + (size_t)row * d;
             float d0 = 0.f, d1 = 0.f;
+#pragma unroll 4
             for (int i = 0; i < d; i += 8) {
                 const float4 qa = *reinterpret_cast<const float4*>(q_lds + i), qb = *reinterpret_cast<const float4*>(q_lds + i + 4);
                 float k8[8];
@@ -250,20 +251,33 @@ void pooled_attention_rows_kernel(const T* __restrict__ q, const T* __restrict__
         l = l * corr + wave_sum(p);
         m = m_new;
         acc[0][0] *= corr; acc[0][1] *= corr; acc[1][0] *= corr; acc[1][1] *= corr;
+        // eight keys at a time: their weights and rows from the lanes that hold them, then the eight loads together, then the sums
         const int n_here = min(TQK_WAVE, n_all - n0);
-        for (int k = 0; k < n_here; ++k) {
-            const float pk = __shfl(p, k, TQK_WAVE);
-            const long long rk = __shfl(row, k, TQK_WAVE);
-            const T* vr = values + (size_t)rk * dv;
+        for (int k = 0; k < n_here; k += 8) {
+            float pk[8];
+            const T* vr[8];
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+                const int kk = min(k + j, n_here - 1);
+                const float pj = __shfl(p, kk, TQK_WAVE);
+                pk[j] = k + j < n_here ? pj : 0.f;
+                vr[j] = values + (size_t)__shfl(row, kk, TQK_WAVE) * dv;
+            }
 #pragma unroll
             for (int c = 0; c < 2; ++c) {
                 const int i = c * 2 * TQK_WAVE + 2 * lane;
                 if (i < dv) {
-                    float v0, v1;
-                    if (sizeof(T) == 2) { const uint32_t vv = *reinterpret_cast<const uint32_t*>(vr + i); v0 = __uint_as_float(vv << 16); v1 = __uint_as_float(vv & 0xffff0000u); }
-                    else { const float2 vv = *reinterpret_cast<const float2*>(vr + i); v0 = vv.x; v1 = vv.y; }
-                    acc[c][0] = fmaf(pk, v0, acc[c][0]);
-                    acc[c][1] = fmaf(pk, v1, acc[c][1]);
+                    float v0[8], v1[8];
+#pragma unroll
+                    for (int j = 0; j < 8; ++j) {
+                        if (sizeof(T) == 2) { const uint32_t vv = *reinterpret_cast<const uint32_t*>(vr[j] + i); v0[j] = __uint_as_float(vv << 16); v1[j] = __uint_as_float(vv & 0xffff0000u); }
+                        else { const float2 vv = *reinterpret_cast<const float2*>(vr[j] + i); v0[j] = vv.x; v1[j] = vv.y; }
+                    }
+#pragma unroll
+                    for (int j = 0; j < 8; ++j) {
+                        acc[c][0] = fmaf(pk[j], v0[j], acc[c][0]);
+                        acc[c][1] = fmaf(pk[j], v1[j], acc[c][1]);
+                    }
                 }
             }
         }

@@ -27,12 +27,12 @@ void streams_fill_kernel(const float* __restrict__ h, float* __restrict__ X, int
 
 // SMAX: the most copies this instance takes (the loops over the copies are unrolled up to it)
 template <typename TY, typename TN, int SMAX>
-__global__ __launch_bounds__(256)
+__global__ __launch_bounds__(1024)
 void streams_step_kernel(float* __restrict__ X, int S, const TY* __restrict__ y, const float* __restrict__ mix, const float* __restrict__ outw,
                          const float* __restrict__ in, const float* __restrict__ nw, const float* __restrict__ nb, float eps,
                          float* __restrict__ u_out, TN* __restrict__ n_out, int W) {
     extern __shared__ float row_u[];
-    __shared__ float scratch[4];
+    __shared__ float scratch[16];
     __shared__ float s_mix[STREAMS_MAX * STREAMS_MAX], s_out[STREAMS_MAX], s_in[STREAMS_MAX];
     const size_t t = blockIdx.x;
     for (int i = threadIdx.x; i < S * S && y; i += blockDim.x) s_mix[i] = mix[i];
@@ -144,7 +144,7 @@ extern "C" int tqk_streams_fill(const float* h, float* X, int n_streams, int n_t
 
 extern "C" int tqk_streams_step(float* X, int n_streams, const void* y, int y_dtype, const float* mix, const float* out_w, const float* in_w,
                                 const float* norm_w, const float* norm_b, float eps, float* u_out, void* n_out, int n_dtype, int n_tokens, int width,
-                                void* stream) {
+                                int wide, void* stream) {
     TQK_REQUIRE(X, "tqk_streams_step: null pointer");
     TQK_REQUIRE(n_streams > 0 && n_streams <= STREAMS_MAX, "tqk_streams_step: %d copies of the stream, the kernel takes up to %d", n_streams, STREAMS_MAX);
     TQK_REQUIRE(!y || (mix && out_w), "tqk_streams_step: an update without its weights");
@@ -154,7 +154,10 @@ extern "C" int tqk_streams_step(float* X, int n_streams, const void* y, int y_dt
     if (n_tokens == 0 || (!y && !in_w)) return 0;
     hipStream_t s = (hipStream_t)stream;
     const size_t lds = (size_t)width * sizeof(float);
-#define TQK_SS_N(TY, TN, SMAX) streams_step_kernel<TY, TN, SMAX><<<n_tokens, 256, lds, s>>>(X, n_streams, (const TY*)y, mix, out_w, in_w, norm_w, norm_b, eps, u_out, (TN*)n_out, width)
+    // wide (steps of few tokens, where the caller does not need one order of a row's sums for every kind of step): four times the
+    // threads a row, so that a thread has a quarter of the loads to wait for one after the other
+    const int threads = wide && width >= 1024 ? 1024 : 256;
+#define TQK_SS_N(TY, TN, SMAX) streams_step_kernel<TY, TN, SMAX><<<n_tokens, threads, lds, s>>>(X, n_streams, (const TY*)y, mix, out_w, in_w, norm_w, norm_b, eps, u_out, (TN*)n_out, width)
 #define TQK_SS(TY, TN) do { if (n_streams <= 1) TQK_SS_N(TY, TN, 1); else if (n_streams <= 2) TQK_SS_N(TY, TN, 2); else if (n_streams <= 4) TQK_SS_N(TY, TN, 4); \
         else if (n_streams <= 8) TQK_SS_N(TY, TN, 8); else TQK_SS_N(TY, TN, STREAMS_MAX); } while (0)
     const int yd = y ? y_dtype : TQK_F32, nd = n_out ? n_dtype : TQK_F32;

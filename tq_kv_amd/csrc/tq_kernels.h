@@ -422,7 +422,8 @@ int tqk_sample(const float* logits, int n_rows, int vocab, float temperature, in
 
 /* The residual stream in several copies, a layer norm with weight and bias, the previous token mixed into a mixer's input (streams.hip).
  * X [tokens, copies, width] float32.  tqk_streams_step: where y is given, X'[t, r] = sum_s mix[s, r] X[t, s] + out_w[r] y[t]; then, where
- * in_w is given, u = sum_s in_w[s] X'[t, s] goes to u_out (if given) and (u - mean) / sqrt(var + eps) norm_w + norm_b to n_out (if given).
+ * in_w is given, u = sum_s in_w[s] X'[t, s] goes to u_out (if given) and (u - mean) / sqrt(var + eps) norm_w + norm_b to n_out (if given);
+ * wide != 0 lets a row have more threads (another order of its sums than with wide == 0).
  * tqk_add_layer_norm: out[i] = that norm of h[rows[i]] + delta[rows[i]] (rows null: row i; h or delta may be null; write_back leaves
  * the sum in h).  tqk_token_shift: out[t] = n[t] + (n[t - 1] - n[t]) mu, with the sequence's state row in place of n[t - 1] for the first
  * token a step brings of it; remember != 0 (steps of one token a sequence) also leaves n[t] in the state.  tqk_shift_remember: the state
@@ -431,7 +432,7 @@ int tqk_streams_max(void);
 int tqk_streams_fill(const float* h, float* X, int n_streams, int n_tokens, int width, void* stream);
 int tqk_streams_step(float* X, int n_streams, const void* y, int y_dtype, const float* mix, const float* out_w, const float* in_w,
                      const float* norm_w, const float* norm_b, float eps, float* u_out, void* n_out, int n_dtype, int n_tokens, int width,
-                     void* stream);
+                     int wide, void* stream);
 int tqk_add_layer_norm(float* h, const void* delta, int delta_dtype, const int32_t* rows, int n_rows, const float* weight, const float* bias,
                        float eps, void* out, int out_dtype, int width, int write_back, void* stream);
 int tqk_token_shift(const float* n, const float* mu, float* state, long long state_stride, const int32_t* tok_seq, const int32_t* tok_pos,
