@@ -59,6 +59,7 @@ MIXERS = [C.parallel(C.left(6, 3, 24, 40, 37, 6, 16, base=40.0, scale=0.3), C.ri
           C.parallel(C.left(4, 4, 10, 14, 64, 64, 0), C.right(2, 6, 10)),
           C.parallel(C.left(8, 2, 64, 64, 130, 8, 64), C.right(4, 64, 64, tau=16.0)),
           C.parallel(C.left(2, 1, 160, 200, 70, 100, 40, scale=0.05), C.right(2, 130, 70)),
+          C.parallel(C.left(2, 2, 32, 64, 33, 5, 16), C.right(1, 32, 32)), C.parallel(C.left(6, 3, 96, 32, 100, 3, 96, scale=0.2), C.right(2, 16, 48)),
           C.retention(3, 24, 20, 16, base=300.0), C.retention(1, 2, 1, 0, decay=[0.5]), C.retention(3, 10, 14, 6), C.retention(4, 128, 128, 128),
           C.retention(2, 200, 136, 64, decay=[0.999, 0.9])]
 
@@ -152,7 +153,7 @@ def test_layer_norm_with_weight_and_bias(dtype, size):
 # ---- whole models ----------------------------------------------------------------------------------------
 _MODELS = {}
 MAKERS = {"mixed": C.config_mixed, "ones": C.config_ones, "plain_residual": C.config_plain_residual,
-          "parallel": lambda: C.config_single("parallel"), "retention": lambda: C.config_single("retention")}
+          "parallel": lambda: C.config_single("parallel"), "retention": lambda: C.config_single("retention", streams=6)}
 
 
 def model(name, tmp_path_factory):
