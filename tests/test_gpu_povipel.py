@@ -404,3 +404,42 @@ def test_greedy_generation_through_the_loop(dtype, tmp_path_factory):
             seq.append(t)
     again = generate(eng, prompts[::-1], params, eos_ids=(), max_batch=2)
     assert again[::-1] == out or dtype == "bfloat16"
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_replay_of_steps_and_the_command_line(dtype, tmp_path_factory):
+    """bin/trace_run fed steps on standard input (a request whole, then its last tokens one by one beside a second request), and bin/tq
+    generate on the same folder: logits and greedy tokens of the plain implementation."""
+    import json
+    import os
+    import subprocess
+    import sys
+    from test_gpu_trace_run import Replay
+    root = os.path.join(os.path.dirname(os.path.abspath(__file__)), "..")
+    cfg = C.config_plain_residual()
+    w = C.weights(cfg, seed=77)
+    folder = C.write_folder(str(tmp_path_factory.mktemp("povipel_replay")), cfg, w)
+    a, b = C.tokens(150, cfg["vocab"], 1), C.tokens(9, cfg["vocab"], 2)
+    want_a, want_b = plain_logits(cfg, w, a), plain_logits(cfg, w, b)
+    r = Replay(folder, dtype, str(tmp_path_factory.mktemp("out")), max_tokens=64 * 6)
+    got = r.step([("x", a, list(range(150)))], end=["x"])
+    close(got.view(-1, cfg["vocab"]), want_a, dtype, "whole")
+    assert r.step([("y", a[:140], []), ("z", b[:5], [])]) is None
+    for t in range(10):
+        live = [("y", [a[140 + t]], [0])] + ([("z", [b[5 + t]], [0])] if t < 4 else [])
+        got = r.step(live, end=(["y"] if t == 9 else []) + (["z"] if t == 3 else [])).view(-1, cfg["vocab"])
+        close(got[0:1], want_a[140 + t:141 + t], dtype, "one by one at %d" % t)
+        if t < 4:
+            close(got[1:2], want_b[5 + t:6 + t], dtype, "the second request at %d" % t)
+    r.finish()
+    if dtype != "float32":
+        return
+    cmd = [sys.executable, os.path.join(root, "bin", "tq"), "--fp32", "generate", folder, "--prompt-ids", ",".join(str(t) for t in b), "-n", "5", "-t", "0",
+           "--repeat-penalty", "1.0", "--json"]
+    out = subprocess.run(cmd, capture_output=True, text=True)
+    assert out.returncode == 0, out.stderr
+    tokens = json.loads(out.stdout.strip().splitlines()[-1])["outputs"][0]
+    seq = list(b)
+    for t in tokens:
+        assert int(plain_logits(cfg, w, seq)[-1].argmax()) == t
+        seq.append(t)
