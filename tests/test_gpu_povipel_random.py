@@ -1,0 +1,89 @@
+"""Povipel configurations drawn from a seed (layers of either mixer in any order, with dense, routed or no feed-forwards, any number of
+copies of the stream, any span and count of passes, windows and blocks of any sizes) through Engine.step against the plain
+implementation: whole prompts, a cut into portions and single tokens, and a batch of two unequal requests."""
+import random
+
+import pytest
+import torch
+
+import plain_povipel as plain
+import povipel_common as C
+from tq_kv_amd import Engine, Model
+
+pytestmark = pytest.mark.gpu
+
+
+def draw(seed):
+    r = random.Random(seed)
+    width = r.choice([48, 64, 96, 160, 192, 256])
+    layers = []
+    for _ in range(r.randint(1, 5)):
+        if r.random() < 0.6:
+            kv = r.choice([1, 2, 3, 4])
+            dim = r.choice([8, 16, 24, 32, 64, 96, 128])
+            left = C.left(kv * r.choice([1, 1, 2, 3, 4, 8]), kv, dim, r.choice([8, 12, 16, 32, 64, 96, 128]), r.choice([1, 3, 16, 40, 64, 100, 136, 200]),
+                          r.choice([1, 2, 3, 4, 8, 16, 30, 64, 70]), r.choice([0, 2, dim // 4 * 2, dim]), base=r.choice([10.0, 500.0, 10000.0, 250000.0]),
+                          scale=r.uniform(0.5, 1.5) / dim ** 0.5)
+            mix = C.parallel(left, C.right(r.choice([1, 2, 3, 6]), r.choice([4, 8, 12, 32, 64]), r.choice([4, 8, 20, 32, 64]), tau=r.choice([1.0, 4.0, 16.0])))
+        else:
+            heads, dim = r.choice([1, 2, 3, 4]), r.choice([4, 8, 12, 32, 64])
+            mix = C.retention(heads, dim, r.choice([4, 8, 20, 32, 64]), r.choice([0, 2, dim // 4 * 2, dim]), base=r.choice([100.0, 1e4, 1e6]),
+                              decay=[1.0 - 2.0 ** -r.uniform(2.0, 10.0) for _ in range(heads)])
+        experts = r.choice([1, 2, 4, 8, 9])
+        mlp = r.choice([None, C.dense(r.choice([24, 64, 100])), C.moe(r.choice([16, 24, 64]), experts, r.randint(1, min(experts, 3)))])
+        layers.append((mix, mlp))
+    n = len(layers)
+    start = r.randint(0, n)
+    stop = r.randint(start, n)
+    loop = r.choice([None, (start, stop, r.randint(1, 3))])
+    return C.config(r.choice([50, 131, 300]), width, layers, streams=r.choice([None, 1, 2, 4, 5, 8]), loop=loop, eps=r.choice([1e-6, 1e-5, 1e-4]),
+                    scale=r.uniform(1.0, 12.0), softcap=r.choice([None, 10.0, 30.0])), r.randint(1, 7)
+
+
+def errors(got, want):
+    got, want = got.float().cpu(), want.float().cpu()
+    d = got - want
+    d = d - d.mean(-1, keepdim=True)
+    return d.pow(2).mean(-1).sqrt() / want.std().clamp_min(1e-6)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("seed", range(16))
+def test_random_configuration(seed, dtype, tmp_path):
+    cfg, rank = draw(seed)
+    w = C.weights(cfg, seed=100 + seed, rank=rank)
+    eng = Engine(Model.from_dir(C.write_folder(str(tmp_path), cfg, w), dtype=dtype), max_tokens=2048, max_slots=4)
+    a, b = C.tokens(290, cfg["vocab"], seed), C.tokens(37, cfg["vocab"], seed + 1)
+    want_a, want_b = plain.forward(cfg, C.as_float(w), a), plain.forward(cfg, C.as_float(w), b)
+
+    def check(got, want, what):
+        e = errors(got, want)
+        assert torch.isfinite(e).all(), what
+        if dtype == "float32":
+            assert e.max().item() <= 3e-4, "%s: row error %.3g at row %d" % (what, e.max().item(), int(e.argmax()))
+        else:       # (a router's close call may send a token to another expert than the plain computation does)
+            assert int((e > 0.12).sum()) <= max(1, e.numel() // 50) and e.max().item() <= 1.0, "%s: the worst row error %.3g" % (what, e.max().item())
+
+    s = eng.open()
+    whole = eng.step([(s, a, list(range(len(a))))])
+    eng.close(s)
+    check(whole, want_a, "whole")
+    # portions beside a second request, then single tokens of both
+    s, t = eng.open(), eng.open()
+    out = [eng.step([(s, a[:200], list(range(200))), (t, b[:30], list(range(30)))])]
+    got_a, got_b = [out[0][:200]], [out[0][200:]]
+    got_a.append(eng.step([(s, a[200:270], list(range(70)))]))
+    for k in range(20):
+        items = [(s, [a[270 + k]], [0])] + ([(t, [b[30 + k]], [0])] if k < 7 else [])
+        o = eng.step(items)
+        got_a.append(o[0:1])
+        if k < 7:
+            got_b.append(o[1:2])
+        if k == 6:
+            eng.close(t)
+    eng.close(s)
+    check(torch.cat(got_a), want_a, "portions and single tokens")
+    check(torch.cat(got_b), want_b, "the second request")
+    if dtype == "float32":
+        assert torch.equal(torch.cat(got_a), whole), "float32 logits depend on the cut or the batch"
+    eng.cache.check()
