@@ -56,13 +56,24 @@ def test_random_configuration(seed, dtype, tmp_path):
     a, b = C.tokens(290, cfg["vocab"], seed), C.tokens(37, cfg["vocab"], seed + 1)
     want_a, want_b = plain.forward(cfg, C.as_float(w), a), plain.forward(cfg, C.as_float(w), b)
 
+    # what rounding alone does: the plain implementation with its products rounded to bfloat16, against float32
+    rounding = {} if dtype == "float32" else {id(x): errors(plain.forward(cfg, C.as_float(w), t, low=torch.bfloat16), x) for t, x in ((a, want_a), (b, want_b))}
+
     def check(got, want, what):
         e = errors(got, want)
         assert torch.isfinite(e).all(), what
         if dtype == "float32":
             assert e.max().item() <= 3e-4, "%s: row error %.3g at row %d" % (what, e.max().item(), int(e.argmax()))
-        else:       # (a router's close call may send a token to another expert than the plain computation does)
-            assert int((e > 0.12).sum()) <= max(1, e.numel() // 50) and e.max().item() <= 1.0, "%s: the worst row error %.3g" % (what, e.max().item())
+            return
+        # A router's close call sends a token to another expert than the float32 computation does; with few experts a token that row's
+        # feed-forward output is another one, and a state carries it to the rows behind it.  The plain implementation in bfloat16 shows
+        # the same rows and sizes, so it is the yardstick: the bulk of the rows as close as its own, not many more rows far off, none
+        # beyond the spread.  float32 is held to every row.
+        r = rounding[id(want)]
+        over, allowed = int((e > 0.12).sum()), 2 * int((r > 0.12).sum()) + max(2, e.numel() // 12)
+        assert e.median().item() <= 2.0 * r.median().item() + 0.02 and over <= allowed and e.max().item() <= max(1.0, 1.5 * r.max().item()), \
+            "%s: median row error %.3g (rounding alone: %.3g), %d rows of %d over (%d), the worst %.3g (%.3g)" % (
+                what, e.median().item(), r.median().item(), over, e.numel(), int((r > 0.12).sum()), e.max().item(), r.max().item())
 
     s = eng.open()
     whole = eng.step([(s, a, list(range(len(a))))])
